@@ -17,7 +17,8 @@ blocks on demand with create / append / seq_len / free calls and status checks
   (both as the attention kernels' operands want them).  Keys and values have pools of their own, so their
   rows may differ in width, and a group whose layers keep one row per position only (``value_dim`` 0) has no
   value pool at all.  A group that keeps a window gives back the pages that have fallen out of every later
-  token's window, so its sequences hold pages for the window only.
+  token's window, so its sequences hold pages for the window only; a group whose tokens see their own chunk of
+  positions only gives back the pages that lie wholly before the chunk of the sequence's next token.
 * The page table of a group, ``[slot][logical page] -> page`` (-1: none), lives on the device and is
   updated only when pages change hands; kernels find a token's rows through its slot.
 * A schedule entry that reads another entry's cache gets a view of that entry's storage and none
@@ -75,6 +76,7 @@ class GroupKey:
     head_dim: int
     value_dim: int
     window: int | None
+    chunk: int | None = None
 
 
 @dataclass
@@ -126,9 +128,12 @@ class CacheGroup:
 
     def first_needed_page(self, length: int) -> int:
         """Lowest logical page that a token at position >= length can still attend to."""
-        if self.key.window is None:
-            return 0
-        return max(0, length - self.key.window + 1) // self.page_size
+        first = 0
+        if self.key.window is not None:
+            first = max(0, length - self.key.window + 1)
+        if self.key.chunk is not None:      # the token at position `length` and all later ones see its chunk's start at the earliest
+            first = max(first, length // self.key.chunk * self.key.chunk)
+        return first // self.page_size
 
     def sync(self) -> None:
         """Sends the rows of the page table that changed to the device.  On a GPU they go through pinned memory
@@ -197,7 +202,7 @@ class PagedCache:
         for e, (cache_need, _state, cache_of) in enumerate(self._needs):
             if cache_need is not None and cache_of is None:
                 by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.value_width,
-                                           cache_need.window), []).append(e)
+                                           cache_need.window, cache_need.chunk), []).append(e)
         # A sequence holds, of a group with a window, the pages that its last `window` positions touch, and during a
         # step those of the step's new positions too, until the step is committed: window + window_step positions
         # lie in at most that many pages plus two.
@@ -226,6 +231,8 @@ class PagedCache:
                     raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of} but their head counts or sizes differ")
                 if src.window is not None and (cache_need.window is None or cache_need.window > src.window):
                     raise CacheError(f"schedule entry {e} looks further back than entry {cache_of}, whose cache it reads, keeps")
+                if src.chunk is not None and cache_need.chunk != src.chunk:
+                    raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of}, which keeps chunks of {src.chunk} positions only")
                 self._entry_group[e] = (g, off, False)
                 self._v_offset[e] = self._v_offset[cache_of]
 
@@ -401,7 +408,7 @@ class PagedCache:
             if any(p < 0 for p in pages):
                 raise CacheError(f"slot {slot} does not hold all pages of its {s.length} positions")
             idx = torch.tensor(pages, dtype=torch.int64, device=self.device)
-            entry = {"first_page": first, "entries": list(g.entries), "key": (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window),
+            entry = {"first_page": first, "entries": list(g.entries), "key": (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk),
                      "keys": g.k_pages.view(-1, g.page_stride)[idx].cpu(), "values": None}
             if g.v_pages is not None:
                 entry["values"] = g.v_pages.view(-1, g.v_page_stride)[idx].cpu()
@@ -415,7 +422,7 @@ class PagedCache:
         if data["page_size"] != self.page_size or len(data["groups"]) != len(self.groups):
             raise CacheError("the saved sequence comes from a cache of another layout")
         for g, d in zip(self.groups, data["groups"]):
-            if tuple(d["key"]) != (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window) or \
+            if tuple(d["key"]) + (None,) * (5 - len(d["key"])) != (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk) or \
                     list(d["entries"]) != list(g.entries) or d["keys"].dtype != self.dtype or \
                     d["keys"].shape[1] != g.page_stride or (d["values"] is None) != (g.v_pages is None):
                 raise CacheError("the saved sequence comes from a cache of another layout")

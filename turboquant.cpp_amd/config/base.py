@@ -95,8 +95,10 @@ class KeyReader:
 
 
 def architecture_name(data: dict) -> str:
-    """The registry key of a config.json: the first entry of ``architectures``."""
+    """The registry key of a config.json: the first entry of ``architectures``, or the string ``architecture``."""
     archs = data.get("architectures")
+    if archs is None and isinstance(data.get("architecture"), str):
+        return data["architecture"]
     if isinstance(archs, str):
         return archs
     if not isinstance(archs, Sequence) or not archs or not isinstance(archs[0], str):

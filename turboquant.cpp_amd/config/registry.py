@@ -21,6 +21,9 @@ class Architecture:
     plan: Callable[[Any], ModelPlan]             # typed configuration -> model plan
     config_to_json: Callable[[Any], dict]        # typed configuration -> dict for config.json
     random_tensors: Callable[..., Any] | None = None   # (config, seed, ...) -> iterator of (name, tensor)
+    # (typed configuration, {tensor name: shape} of the checkpoint) -> typed configuration, for designs that leave
+    # sizes to the shapes of their tensors
+    complete: Callable[[Any, dict], Any] | None = None
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}

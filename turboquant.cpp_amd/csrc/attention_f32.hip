@@ -22,6 +22,7 @@
 // column l%16, rows 4*(l/16) + v, v<4.  A lane's 16 bytes of an operand row are 4 consecutive elements of the
 // contraction, used one by one by four instructions.
 #include "common.h"
+#include "score_mod.h"
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -43,6 +44,7 @@ struct AttnF32Args {
   float* out;              // [T][nh][hd]
   float* partial;          // decode: [B][nh][tiles][hd + 2]
   int tiles_max;           // decode: tiles per sequence in `partial`
+  ScoreMod mod;            // what happens to a score before the softmax, and the chunks of positions (score_mod.h)
 };
 
 // Lanes l and l ^ 8 (the same quarter g = l / 16, rows r and r ^ 8 of 16) fetched whole lines: lane (r, g) chunk
@@ -73,6 +75,7 @@ __device__ __forceinline__ float group_sum(float v) {
 // update, and the product with the values from `vf` (value operand of d-tile dt, subtile kt).
 template <int ND, class KF, class VF>
 __device__ __forceinline__ void attend_tile(const f32x4 (&qf)[ND], KF kf, VF vf, int key0, int pos_q, int lo_q, float scale,
+                                            float cap, bool biased, float r1, float r2,
                                             float& m_run, float& l_run, f32x4 (&acc)[ND]) {
   const int g = (threadIdx.x % 64) / 16;
   f32x4 s[4];
@@ -92,7 +95,7 @@ __device__ __forceinline__ void attend_tile(const f32x4 (&qf)[ND], KF kf, VF vf,
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int j = key0 + 16 * kt + 4 * g + v;
-      const float x = (j <= pos_q && j >= lo_q) ? s[kt][v] * scale : -INFINITY;
+      const float x = (j <= pos_q && j >= lo_q) ? mod_score(s[kt][v] * scale, cap, biased, r1, r2, pos_q - j) : -INFINITY;
       s[kt][v] = x;
       m_tile = fmaxf(m_tile, x);
     }
@@ -147,7 +150,9 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
   const int qi = blk * 64 + wave * 16 + r;
   const bool q_ok = qi < n_new;
   const int pos_q = q_ok ? start + qi : -1;
-  const int lo_q = p.window > 0 ? max(0, pos_q - p.window + 1) : 0;
+  const int lo_q = reach_lo(pos_q, p.window, p.mod.chunk);
+  const bool biased = p.mod.r1 != nullptr;
+  const float r1 = biased ? p.mod.r1[h] : 0.f, r2 = biased ? p.mod.r2[h] : 0.f;
   f32x4 qf[ND];
   const float* qrow = p.q + ((size_t)(t0 + (q_ok ? qi : 0)) * p.nh + h) * hd;
 #pragma unroll
@@ -162,9 +167,9 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
 
   // what the block as a whole can reach, and what this wave can
   const int blk_first = start + blk * 64, blk_last = start + min(n_new, blk * 64 + 64) - 1;
-  const int blk_lo = p.window > 0 ? max(0, blk_first - p.window + 1) : 0;
+  const int blk_lo = reach_lo(blk_first, p.window, p.mod.chunk);
   const int wave_first = start + blk * 64 + wave * 16, wave_last = min(blk_last, wave_first + 15);
-  const int wave_lo = p.window > 0 ? max(0, wave_first - p.window + 1) : 0;
+  const int wave_lo = reach_lo(wave_first, p.window, p.mod.chunk);
 
   for (int tile = blk_lo / AT; tile * AT <= blk_last; ++tile) {
     const int key0 = tile * AT;
@@ -189,7 +194,7 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
     attend_tile<ND>(
         qf, [&](int kt, int u) { return *reinterpret_cast<const f32x4*>(&Ks[(16 * kt + r) * KLD + 16 * u + 4 * g]); },
         [&](int dt, int kt) { return *reinterpret_cast<const f32x4*>(&Vt[(16 * dt + r) * VLD + 16 * kt + 4 * g]); },
-        key0, pos_q, lo_q, p.scale, m_run, l_run, acc);
+        key0, pos_q, lo_q, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
   }
   if (!q_ok) return;
   const float inv = 1.0f / l_run;
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
   const int b = blockIdx.x, kvh = blockIdx.y / passes, pass = blockIdx.y % passes;
   const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
   const int pos = p.start[b];                       // the token's position: it attends to lo..pos
-  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int lo = reach_lo(pos, p.window, p.mod.chunk);
   const int first = lo / AT, last = pos / AT;
   const int tile = first + blockIdx.z;
   if (tile > last) return;
@@ -226,6 +231,8 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
   const int hq = pass * 16 + r;                     // this lane's query: head hq of the group
   const bool q_ok = hq < group;
   const int h = kvh * group + (q_ok ? hq : 0);
+  const bool biased = p.mod.r1 != nullptr;
+  const float r1 = biased ? p.mod.r1[h] : 0.f, r2 = biased ? p.mod.r2[h] : 0.f;
   const int t = p.cu_seqlens[b];
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   f32x4 qf[ND];
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
             v_next = t1;
             return t0;
           },
-          key0, q_ok ? pos : -1, lo, p.scale, m_run, l_run, acc);
+          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
     } else {
       // (what lies beyond the head size is asked for at the tile's first address instead and replaced by zeros:
       // every lane loads, so that no load waits behind a branch)
@@ -285,7 +292,7 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
                 reinterpret_cast<const f32x4*>(d < hd ? vp + (size_t)d * p.page_size + 16 * kt + 4 * g : vp));
             return d < hd ? x : zero;
           },
-          key0, q_ok ? pos : -1, lo, p.scale, m_run, l_run, acc);
+          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
     }
     if (!q_ok) return;
     float* out = p.partial + (((size_t)b * p.nh + h) * p.tiles_max + tile) * (hd + 2);
@@ -312,7 +319,7 @@ __global__ __launch_bounds__(64) void attn_f32_join_kernel(AttnF32Args p) {
   __shared__ float wgt[F32_JOIN_TILES];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int pos = p.start[b];
-  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int lo = reach_lo(pos, p.window, p.mod.chunk);
   const int first = lo / AT, last = pos / AT;
   const int stride = p.hd + 2;
   const float* part = p.partial + ((size_t)b * p.nh + h) * p.tiles_max * stride;
@@ -353,7 +360,8 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
     const int tiles = (max_end + AT - 1) / AT;
     const int group = p.nh / p.nkv, passes = (group + 15) / 16;
     // with a window a token reaches at most window positions, which lie in window / AT + 2 tiles at the most
-    const int waves = p.window > 0 ? min(tiles, p.window / AT + 2) : tiles;
+    int waves = p.window > 0 ? min(tiles, p.window / AT + 2) : tiles;
+    if (p.mod.chunk > 0) waves = min(waves, p.mod.chunk / AT + 2);      // and a chunk in chunk / AT + 2
     if (p.nkv * passes > 65535 || waves > 65535 || tiles > F32_JOIN_TILES) return TQ_ERR_UNSUPPORTED;
     // whole lines only where the head fills its tiles of 16 (32, 64, 128, 256): the loads of that form have no
     // guard on the head size, and a head of 96 would read beyond its rows and, in the last page, beyond the pool
@@ -381,11 +389,14 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
 // The tokens are runs of consecutive positions, one per sequence (cu_seqlens, slots, start as in AttnF32Args);
 // decode: every run is one token and `partial` holds tq_attention_f32_scratch(B, nh, hd, max_end) floats.
 // hd must be a multiple of 4 and at most 256, page_size a multiple of 64, page_stride a multiple of 4.
-TQ_API int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
-                            const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
-                            int B, int nh, int nkv, int hd, int window, float scale, void* out, void* partial, int decode,
-                            int max_new, int max_end, hipStream_t st) {
+// softcap, r1, r2, chunk: see score_mod.h (0, null, null, 0: nothing).
+TQ_API int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+                                const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
+                                int B, int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1,
+                                const float* r2, int chunk, void* out, void* partial, int decode, int max_new,
+                                int max_end, hipStream_t st) {
   if (B <= 0) return 0;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
   if (hd <= 0 || hd % 4 != 0 || hd > 256 || nkv <= 0 || nh % nkv != 0 || page_size % AT != 0 || page_stride % 4 != 0)
     return TQ_ERR_UNSUPPORTED;
   if (((size_t)q | (size_t)k_pool | (size_t)v_pool | (size_t)out) & 15) return TQ_ERR_UNSUPPORTED;
@@ -393,7 +404,7 @@ TQ_API int tq_attention_f32(const void* q, const void* k_pool, const void* v_poo
   if (max_new <= 0 || max_end <= 0) return TQ_ERR_BAD_ARG;
   AttnF32Args p{(const float*)q, (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, cu_seqlens, slots,
                 start, page_size, page_stride, nh, nkv, hd, window, scale, (float*)out, (float*)partial,
-                (max_end + AT - 1) / AT};
+                (max_end + AT - 1) / AT, ScoreMod{softcap, r1, r2, chunk}};
   int rc;
   if (hd <= 16) rc = launch_attention_f32<1>(p, B, decode, max_new, max_end, st);
   else if (hd <= 32) rc = launch_attention_f32<2>(p, B, decode, max_new, max_end, st);
@@ -403,4 +414,13 @@ TQ_API int tq_attention_f32(const void* q, const void* k_pool, const void* v_poo
   if (rc) return rc;
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+                            const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
+                            int B, int nh, int nkv, int hd, int window, float scale, void* out, void* partial, int decode,
+                            int max_new, int max_end, hipStream_t st) {
+  return tq_attention_f32_mod(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride,
+                              B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, partial, decode, max_new,
+                              max_end, st);
 }

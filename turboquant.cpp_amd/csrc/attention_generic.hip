@@ -11,6 +11,7 @@
 // has been written for all tokens of the step before it runs.  In a page, keys lie [kv head][row][hd]
 // and values transposed, [kv head][hd][row].
 #include "common.h"
+#include "score_mod.h"
 
 #define CHUNK 128
 
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
     const act_t* __restrict__ q, const act_t* __restrict__ k_pool, const act_t* __restrict__ v_pool,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int bt_stride, int page_size, int64_t page_stride, int nh, int nkv, int hd, int window, float scale,
-    act_t* __restrict__ out) {
+    ScoreMod mod, act_t* __restrict__ out) {
   extern __shared__ float sm[];
   float* qs = sm;                       // hd
   float* ps = qs + hd;                  // CHUNK probabilities
@@ -29,7 +30,9 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
   const int kvh = h / (nh / nkv);
   const int pos = positions[t];
   const int* table = block_table + (size_t)seq_of_token[t] * bt_stride;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = reach_lo(pos, window, mod.chunk);
+  const bool biased = mod.r1 != nullptr;
+  const float r1 = biased ? mod.r1[h] : 0.f, r2 = biased ? mod.r2[h] : 0.f;
 
   for (int i = tid; i < hd; i += CHUNK) qs[i] = to_f32(q[((size_t)t * nh + h) * hd + i]);
   __syncthreads();
@@ -49,7 +52,7 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
       const act_t* kr = k_pool + off + (int64_t)(j % page_size) * hd;   // keys: [row][hd]
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
-      sc = d * scale;
+      sc = mod_score(d * scale, mod.cap, biased, r1, r2, pos - j);
     }
     head_off[tid] = off;
     row_in_page[tid] = j % page_size;
@@ -85,17 +88,30 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
   }
 }
 
-TQ_API int tq_attention_generic(const void* q, const void* k_pool, const void* v_pool, const int* positions,
-                                const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
-                                int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
-                                void* out, hipStream_t st) {
+// softcap, r1, r2, chunk: what happens to a score before the softmax and the chunks of positions, see score_mod.h
+// (0, null, null, 0: nothing).
+TQ_API int tq_attention_generic_mod(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+                                    const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
+                                    int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
+                                    float softcap, const float* r1, const float* r2, int chunk, void* out,
+                                    hipStream_t st) {
   if (T <= 0) return 0;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
+  const ScoreMod mod{softcap, r1, r2, chunk};
   if (hd > 4 * CHUNK || nkv <= 0 || nh % nkv != 0) return TQ_ERR_UNSUPPORTED;
   if (nh > 65535) return TQ_ERR_UNSUPPORTED;
   const size_t shmem = (size_t)(hd + CHUNK + 4) * sizeof(float) + CHUNK * (sizeof(int64_t) + sizeof(int));
   hipLaunchKernelGGL(attention_generic_kernel, dim3(T, nh), dim3(CHUNK), shmem, st, (const act_t*)q,
                      (const act_t*)k_pool, (const act_t*)v_pool, positions, seq_of_token, block_table, bt_stride,
-                     page_size, page_stride, nh, nkv, hd, window, scale, (act_t*)out);
+                     page_size, page_stride, nh, nkv, hd, window, scale, mod, (act_t*)out);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_attention_generic(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+                                const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
+                                int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
+                                void* out, hipStream_t st) {
+  return tq_attention_generic_mod(q, k_pool, v_pool, positions, seq_of_token, block_table, bt_stride, page_size,
+                                  page_stride, T, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, st);
 }

@@ -21,6 +21,7 @@
 // multiples of 64 positions and runs at multiples of the run length, so the order of every sum depends only on
 // the token's own position.
 #include "common.h"
+#include "score_mod.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -59,7 +60,30 @@ struct AttnArgs {
   bf16_t* out;                  // [T][nh][hd]
   float* partial;               // decoding: [B][nh][max_runs][hd + 2]
   int max_runs;
+  ScoreMod mod;                 // what happens to a score before the softmax, and the chunks of positions (score_mod.h)
 };
+
+// What softmax_tile needs of the score's changes for the QG groups of columns a lane holds: the plain scale, the cap and
+// each column's pair of the distance bias (a column is a token of one head in prompts, a head in decoding).
+template <int QG, bool MOD>
+struct ColMod {
+  bool biased;
+  float scale, cap;
+  float r1[QG], r2[QG];
+};
+template <int QG, bool MOD>
+__device__ __forceinline__ ColMod<QG, MOD> col_mod(const AttnArgs& a, const int (&head)[QG]) {
+  ColMod<QG, MOD> m;
+  m.biased = MOD && a.mod.r1 != nullptr;
+  m.scale = a.scale;
+  m.cap = a.mod.cap;
+#pragma unroll
+  for (int g = 0; g < QG; ++g) {
+    m.r1[g] = m.biased ? a.mod.r1[head[g]] : 0.f;
+    m.r2[g] = m.biased ? a.mod.r2[head[g]] : 0.f;
+  }
+  return m;
+}
 
 __device__ __forceinline__ bf16x8 ld16(const bf16_t* p) {
   const uint4 v = *reinterpret_cast<const uint4*>(p);
@@ -118,11 +142,25 @@ __device__ __forceinline__ int v_swz(int d, int ch) { return d * TILE + ((ch ^ (
 // The part of a tile between its two products, for QG groups of 16 columns: s holds the tile's scores (rows of
 // block jt as tile_step says); afterwards m_run, l_run and o are brought to the new running maximum and pf holds the
 // probabilities 2^(s * scale2 - m) as the operand of the second product.
-template <int DT, int QG>
+template <int DT, int QG, bool MOD>
 __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
                                              int pos0, const int (&p_q)[QG], const int (&lo_q)[QG], float scale2,
-                                             bool masked, bf16x8 (&pf)[2][QG]) {
+                                             bool masked, bf16x8 (&pf)[2][QG], const ColMod<QG, MOD>& cm) {
   const int c = (threadIdx.x % 64) / 16;
+  if constexpr (MOD) {
+    // a cap or a distance bias: the scores are brought to their final value in natural units here, and only the
+    // change of base is left to the factor below
+#pragma unroll
+    for (int g = 0; g < QG; ++g)
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
+          s[g][jt][v] = mod_score(s[g][jt][v] * cm.scale, cm.cap, cm.biased, cm.r1[g], cm.r2[g], p_q[g] - key);
+        }
+    scale2 = LOG2E;
+  }
   // mask, running maximum, probabilities
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
@@ -186,11 +224,11 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][D
 // bytes, eight lanes to a row, and lanes l and l ^ 8 exchange what belongs to the other's row.
 // scale2 = scale * log2(e) > 0: maxima are kept in that unit and probabilities are 2^(s * scale2 - m), which is
 // exp(s * scale - max) with one instruction for the power.
-template <int DT, int QG, bool EXACT, bool SWZ = false, bool ONCE = false>
+template <int DT, int QG, bool EXACT, bool SWZ = false, bool ONCE = false, bool MOD = false>
 __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
                                           const bf16x8 (&qf)[QG][(DT + 1) / 2], const bf16_t* kt, int k_stride,
                                           const bf16_t* vt, int v_stride, int hd, int pos0, const int (&p_q)[QG],
-                                          const int (&lo_q)[QG], float scale2, bool masked) {
+                                          const int (&lo_q)[QG], float scale2, bool masked, const ColMod<QG, MOD>& cm) {
   constexpr int KS = (DT + 1) / 2;
   const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
   // EXACT: hd == 16 DT with DT even, so nothing below depends on hd and every product is unconditional
@@ -232,7 +270,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     }
   }
   bf16x8 pf[2][QG];
-  softmax_tile<DT, QG>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf);
+  softmax_tile<DT, QG, MOD>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf, cm);
   if (ONCE) {
     // a row of values (64 positions of one dimension) is one line: both halves of the tile come with it
 #pragma unroll
@@ -261,11 +299,11 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 }
 
 // Runs the wave's 16 columns over tiles [tile_beg, tile_end) straight from the cache pages.
-template <int DT, bool EXACT>
+template <int DT, bool EXACT, bool MOD>
 __device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
                                        const bf16x8 (&qf)[1][(DT + 1) / 2], const bf16_t* kh, const bf16_t* vh,
                                        const int* table, int page_size, int64_t page_stride, int hd, int tile_beg,
-                                       int tile_end, int p, bool valid, int lo_q, float scale2) {
+                                       int tile_end, int p, bool valid, int lo_q, float scale2, const ColMod<1, MOD>& cm) {
   const int pq[1] = {valid ? p : -1}, lq[1] = {lo_q};
   for (int tile = tile_beg; tile < tile_end; ++tile) {
     const int pos0 = tile * TILE;
@@ -274,7 +312,7 @@ __device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], flo
     const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
     const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
     const bool masked = pos0 + TILE - 1 > p || pos0 < lo_q;      // the same for all lanes
-    tile_step<DT, 1, EXACT, false, EXACT>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked);
+    tile_step<DT, 1, EXACT, false, EXACT, MOD>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked, cm);
   }
 }
 
@@ -306,10 +344,11 @@ __device__ __forceinline__ void fetch_tile(TileRegs<DT>& t, const bf16_t* kt, in
     t.v[dt][1] = ld16_once(vt + (16 * dt + 8 + r8) * v_stride + q8);
   }
 }
-template <int DT>
+template <int DT, bool MOD>
 __device__ __forceinline__ void tile_step_regs(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
                                                const bf16x8 (&qf)[1][DT / 2], TileRegs<DT>& t, int pos0,
-                                               const int (&p_q)[1], const int (&lo_q)[1], float scale2, bool masked) {
+                                               const int (&p_q)[1], const int (&lo_q)[1], float scale2, bool masked,
+                                               const ColMod<1, MOD>& cm) {
   f32x4 s[1][4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) {
@@ -321,7 +360,7 @@ __device__ __forceinline__ void tile_step_regs(f32x4 (&o)[1][DT], float (&m_run)
       s[0][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.k[jt][ks]), qf[0][ks], s[0][jt], 0, 0, 0);
   }
   bf16x8 pf[2][1];
-  softmax_tile<DT, 1>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf);
+  softmax_tile<DT, 1, MOD>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf, cm);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     to_own_row(t.v[dt][0], t.v[dt][1]);
@@ -329,11 +368,11 @@ __device__ __forceinline__ void tile_step_regs(f32x4 (&o)[1][DT], float (&m_run)
     o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.v[dt][1]), pf[1][0], o[0][dt], 0, 0, 0);
   }
 }
-template <int DT>
+template <int DT, bool MOD>
 __device__ __forceinline__ void attend_ahead(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
                                              const bf16x8 (&qf)[1][DT / 2], const bf16_t* kh, const bf16_t* vh,
                                              const int* table, int page_size, int64_t page_stride, int tile_beg,
-                                             int tile_end, int p, bool valid, int lo_q, float scale2) {
+                                             int tile_end, int p, bool valid, int lo_q, float scale2, const ColMod<1, MOD>& cm) {
   constexpr int hd = 16 * DT;
   const int pq[1] = {valid ? p : -1}, lq[1] = {lo_q};
   TileRegs<DT> t0, t1;
@@ -348,7 +387,7 @@ __device__ __forceinline__ void attend_ahead(f32x4 (&o)[1][DT], float (&m_run)[1
   do {                                                                                                     \
     const int pos0_ = (tile) * TILE;                                                                       \
     const bool masked_ = pos0_ + TILE - 1 > p || pos0_ < lo_q;                                             \
-    tile_step_regs<DT>(o, m_run, l_run, qf, regs, pos0_, pq, lq, scale2, masked_);                         \
+    tile_step_regs<DT, MOD>(o, m_run, l_run, qf, regs, pos0_, pq, lq, scale2, masked_, cm);                     \
   } while (0)
   TQ_FETCH_TILE(t0, tile_beg);
   for (int tile = tile_beg; tile < tile_end; tile += 2) {
@@ -383,7 +422,7 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 #define KPAD 8
 #define VSTR 72
 
-template <int DT, int QG, bool EXACT>
+template <int DT, int QG, bool EXACT, bool MOD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int QW = 16 * QG;
@@ -416,7 +455,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int qi = qb + wave * QW + g * 16 + r;
     const bool valid = qi < n;
     p_q[g] = valid ? start + qi : -1;
-    lo_q[g] = a.window > 0 ? max(0, p_q[g] - a.window + 1) : 0;
+    lo_q[g] = reach_lo(p_q[g], a.window, a.mod.chunk);
     load_query<DT>(qf[g], a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * hd, hd, valid);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -425,12 +464,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   }
   // tiles the workgroup goes through, and those among them that this wave's tokens can see
   const int wg_first = start + qb, wg_last = start + min(qb + 4 * QW, n) - 1;
-  const int tile_beg = (a.window > 0 ? max(0, wg_first - a.window + 1) : 0) / TILE, tile_end = wg_last / TILE + 1;
+  const int tile_beg = reach_lo(wg_first, a.window, a.mod.chunk) / TILE, tile_end = wg_last / TILE + 1;
   const int wq0 = qb + wave * QW;
   const bool wave_has = wq0 < n;
   const int wave_first = start + wq0, wave_last = start + min(wq0 + QW, n) - 1;
-  const int wave_lo_last = a.window > 0 ? max(0, wave_last - a.window + 1) : 0;     // first key of the wave's last token
-  const int wave_beg = (a.window > 0 ? max(0, wave_first - a.window + 1) : 0) / TILE;
+  const int wave_lo_last = reach_lo(wave_last, a.window, a.mod.chunk);     // first key of the wave's last token
+  const int wave_beg = reach_lo(wave_first, a.window, a.mod.chunk) / TILE;
+  int heads_g[QG];
+#pragma unroll
+  for (int g = 0; g < QG; ++g) heads_g[g] = h;
+  const ColMod<QG, MOD> cm = col_mod<QG, MOD>(a, heads_g);
   const int wave_end = wave_has ? wave_last / TILE + 1 : 0;
 
   // what this thread carries of every tile: where its chunks lie in the tile in memory and in LDS (a thread
@@ -480,8 +523,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     if (tile >= wave_beg && tile < wave_end) {
       const int pos0 = tile * TILE;
       const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
-      tile_step<DT, QG, EXACT, EXACT>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
-                                      a.scale * LOG2E, masked);
+      tile_step<DT, QG, EXACT, EXACT, false, MOD>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
+                                      a.scale * LOG2E, masked, cm);
     }
     __syncthreads();
   }
@@ -513,14 +556,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // that no wave has more than one or two of them (left to the last wave alone, 30 runs in a row made a step with
 // one sequence beyond position 4096 and seven shorter ones a third slower).
 // AHEAD (with EXACT): the form for steps of few waves, which fetches a tile ahead (attend_ahead).
-template <int DT, bool EXACT, bool AHEAD = false>
+template <int DT, bool EXACT, bool AHEAD = false, bool MOD = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.z;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
   const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
   const int lane = threadIdx.x, r = lane % 16, c = lane / 16;
   const int p = a.start[b];
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int lo = reach_lo(p, a.window, a.mod.chunk);
   const int S = tiles_per_run(p), n_runs = runs_at(p);
   if ((int)blockIdx.x >= n_runs) return;
   const int hg = cg * 16 + r;                 // head within the group
@@ -529,6 +572,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : 
   const int64_t head_off = (int64_t)kvh * a.page_size * a.hd;
   const int* table = a.block_table + (size_t)a.slots[b] * a.bt_stride;
   const int t = a.cu_seqlens[b];
+  const int head1[1] = {h};
+  const ColMod<1, MOD> cm = col_mod<1, MOD>(a, head1);
 
   bf16x8 qf[1][(DT + 1) / 2];
   load_query<DT>(qf[0], a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
@@ -540,11 +585,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : 
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
     if constexpr (AHEAD)
-      attend_ahead<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                       tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
+      attend_ahead<DT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                       tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm);
     else
-      attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
+      attend<DT, EXACT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm);
     if (!valid) continue;
     float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
@@ -569,7 +614,7 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
   __shared__ float wgt[MAX_RUNS_LDS];
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const int p = a.start[b];
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int lo = reach_lo(p, a.window, a.mod.chunk);
   const int S = tiles_per_run(p);
   const int run_beg = lo / TILE / S, run_end = p / TILE / S + 1;
   const int stride = a.hd + 2;
@@ -611,27 +656,38 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------ launch
-template <int DT, int QG, bool EXACT>
-static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
+template <int DT, int QG, bool EXACT, bool MOD>
+static int launch_prefill_as(const AttnArgs& a, int B, int max_new, hipStream_t st) {
   const size_t shmem = 2 * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT, MOD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
   if ((int64_t)n_blocks * a.nh * B > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);
+  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT, MOD>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);
   return 0;
 }
-template <int DT, bool EXACT>
-static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
+// (the kernels that cap or bias scores are instantiations of their own, so that the others carry nothing of it)
+template <int DT, int QG, bool EXACT>
+static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
+  return (a.mod.cap > 0.f || a.mod.r1) ? launch_prefill_as<DT, QG, EXACT, true>(a, B, max_new, st)
+                                       : launch_prefill_as<DT, QG, EXACT, false>(a, B, max_new, st);
+}
+template <int DT, bool EXACT, bool MOD>
+static void launch_decode_as(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
   const int g = a.nh / a.nkv;
   const dim3 grid(grid_runs, a.nkv * ((g + 15) / 16), B);
   // at most a wave to a SIMD: each has the registers to fetch a tile ahead (one sequence at position 8,191: 2.38 ms a
   // step against 2.61; with more waves than that the form is no faster, from twice as many on slower)
   if (EXACT && DT <= 8 && (int64_t)grid.x * grid.y * grid.z <= 1024)
-    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, EXACT && DT <= 8>), grid, dim3(64), 0, st, a);
+    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, EXACT && DT <= 8, MOD>), grid, dim3(64), 0, st, a);
   else
-    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), grid, dim3(64), 0, st, a);
+    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, false, MOD>), grid, dim3(64), 0, st, a);
   hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
+}
+template <int DT, bool EXACT>
+static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
+  if (a.mod.cap > 0.f || a.mod.r1) launch_decode_as<DT, EXACT, true>(a, B, grid_runs, st);
+  else launch_decode_as<DT, EXACT, false>(a, B, grid_runs, st);
 }
 
 // Number of floats of `partial` that decoding B sequences up to position max_end needs.
@@ -641,18 +697,21 @@ TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
 
 // decode != 0: every sequence brings exactly one token.  max_new: longest run of new tokens of a sequence;
 // max_end: largest position + 1 that any token of the step has.
-TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                             int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
-                             int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale, void* out,
-                             float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+// softcap, r1, r2, chunk: see score_mod.h (0, null, null, 0: nothing).
+TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                                 int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                                 int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
+                                 float softcap, const float* r1, const float* r2, int chunk, void* out,
+                                 float* partial, int decode, int max_new, int max_end, hipStream_t st) {
   if (B <= 0) return 0;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
   if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
   if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
-             most_runs(max_end)};
+             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk}};
   const int dt = hd / 16;
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
@@ -679,4 +738,13 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
   }
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                             int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                             int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale, void* out,
+                             float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+  return tq_attention_mfma_mod(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride,
+                               B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, partial, decode, max_new,
+                               max_end, st);
 }

@@ -18,13 +18,13 @@ CSRC = os.path.dirname(os.path.abspath(__file__))
 
 # sources per activation type: each has matrix-core kernels of its own
 # (host/: the step executor and its way into the vendor's matrix library, host code that calls the kernels' entry points)
-COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip",
+COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip", "delta_rule.hip",
                   "host/engine.cpp", "host/vendor.cpp"]
 SOURCES = {
     "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
-HEADERS = ["common.h", "gates.def", "no_alloc.h", "gemm_mfma.h", "turboquant_kernels.h", "host/engine.h", "host/vendor.h",
+HEADERS = ["common.h", "score_mod.h", "gates.def", "no_alloc.h", "gemm_mfma.h", "turboquant_kernels.h", "host/engine.h", "host/vendor.h",
            "host/host_common.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",

@@ -1,0 +1,301 @@
+// The gated delta rule with one decay per head and key channel, over per-sequence state of fixed size.
+//
+// Per head, with a state S [D][V] (key channels by value channels) that starts at zero, token by token:
+//   S <- diag(g) S ;  u = beta (v - S^T k) ;  S <- S + k u^T ;  o = S^T q
+// with g = exp(-exp(A_log_h) * softplus(a + dt_bias)) in (0, 1) per key channel, beta = sigmoid(b) per head, and q, k
+// unit vectors per head (q also times D^-1/2) made from projections that passed a short causal convolution over time
+// and silu.  Each head's o is then divided by its root mean square, multiplied by a weight per value channel and by a
+// sigmoid gate.  Everything here is float arithmetic on both libraries; the products around it are the library's.
+//
+// Three kernels, for prompts and for decoding alike (a decoded token is a run of one):
+//   delta_prep   per token: convolution (its first inputs from the sequence's state), silu, unit vectors, beta, and
+//                the low-rank activations of the decay and the gate in the activation type, for the product behind
+//   delta_scan   per (sequence, head, block of value channels): the recurrence over the run's tokens in order, the
+//                state in registers (16 key channels of one value channel per lane), tokens staged through LDS in
+//                chunks with their decays worked out in parallel
+//   delta_out    per token: norm and gate of every head; and per sequence: the convolution's new state
+//
+// A sequence's row of state (float): S as [H][D][V], then for every convolution channel (q's, k's, v's) its last
+// taps - 1 inputs, oldest first.  Projections P [T][NP] (float): q (G D) | k (G D) | v (H V) | b (H) | a1 (ra) | g1 (rg).
+#include "common.h"
+
+#define DR_ROWS 16        // key channels of a value channel that one lane keeps
+#define DR_CHUNK 16       // tokens staged at a time
+
+struct DeltaDims {
+  int H, G, D, V;         // heads, q/k heads, key width, value width
+  int taps;               // of the convolution
+  int ra, rg;             // ranks of the decay's and the gate's first product
+};
+__host__ __device__ __forceinline__ int dd_channels(const DeltaDims& d) { return 2 * d.G * d.D + d.H * d.V; }
+__host__ __device__ __forceinline__ int dd_np(const DeltaDims& d) { return dd_channels(d) + d.H + d.ra + d.rg; }
+__host__ __device__ __forceinline__ int64_t dd_state(const DeltaDims& d) {
+  return (int64_t)d.H * d.D * d.V + (int64_t)dd_channels(d) * (d.taps - 1);
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// ------------------------------------------------------------------------------------------ per token
+// grid (T), block 256: a wave takes the "units" of its token in turn: the G query heads, the G key heads, the H
+// value heads, and one unit for beta and the low-rank activations.  An input before the token's run comes from the
+// state: the token is the c-th of its run if c of the taps - 1 tokens before it in the packed arrays have its slot
+// (c < taps - 1), and then input i - d (d > c) is the state's (d - c)-th most recent.
+__global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict__ P, const int* __restrict__ slot_of_token,
+                                                         const float* __restrict__ state, int64_t state_stride,
+                                                         const float* __restrict__ conv_w, DeltaDims dm,
+                                                         float* __restrict__ qn, float* __restrict__ kn,
+                                                         float* __restrict__ vc, float* __restrict__ beta,
+                                                         act_t* __restrict__ low) {
+  const int t = blockIdx.x, wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int G = dm.G, D = dm.D, H = dm.H, V = dm.V, K = dm.taps;
+  const int NP = dd_np(dm), C = dd_channels(dm);
+  const int slot = slot_of_token[t];
+  int before = 0;        // tokens of the same run right before this one, up to taps - 1
+  while (before < K - 1 && t - before - 1 >= 0 && slot_of_token[t - before - 1] == slot) ++before;
+  const float* hist = state + (size_t)slot * state_stride + (size_t)H * D * V;      // [C][K - 1]
+  const float* row = P + (size_t)t * NP;
+  const int units = 2 * G + H + 1;
+  for (int u = wave; u < units; u += 4) {
+    if (u == units - 1) {
+      for (int h = lane; h < H; h += TQ_WAVE) beta[(size_t)t * H + h] = sigmoid_f(row[C + h]);
+      for (int i = lane; i < dm.ra + dm.rg; i += TQ_WAVE)
+        low[(size_t)t * (dm.ra + dm.rg) + i] = from_f32<act_t>(row[C + H + i]);
+      continue;
+    }
+    const bool is_v = u >= 2 * G;
+    const int width = is_v ? V : D;
+    const int c0 = is_v ? 2 * G * D + (u - 2 * G) * V : u * D;      // the unit's first channel
+    float ss = 0.f;
+    // (a unit wider than 64 goes in turns; its values wait in the output and are scaled afterwards)
+    float* dst = is_v ? vc + (size_t)t * H * V + (size_t)(u - 2 * G) * V
+                      : (u < G ? qn + (size_t)t * G * D + (size_t)u * D : kn + (size_t)t * G * D + (size_t)(u - G) * D);
+    for (int i = lane; i < width; i += TQ_WAVE) {
+      const int c = c0 + i;
+      const float* w = conv_w + (size_t)c * K;
+      float y = 0.f;
+      for (int j = 0; j < K; ++j) {
+        const int d = K - 1 - j;        // how many tokens back
+        const float in = d <= before ? P[(size_t)(t - d) * NP + c] : hist[(size_t)c * (K - 1) + (K - 1) - (d - before)];
+        y = fmaf(w[j], in, y);
+      }
+      y = silu_f(y);
+      dst[i] = y;
+      ss += y * y;
+    }
+    if (is_v) continue;
+    ss = wave_sum(ss);
+    const float f = (1.0f / sqrtf(ss + 1e-6f)) * (u < G ? 1.0f / sqrtf((float)D) : 1.0f);
+    for (int i = lane; i < width; i += TQ_WAVE) dst[i] *= f;
+  }
+}
+
+// ------------------------------------------------------------------------------------------ the recurrence
+// grid (H * col_blocks, B), block NSEG * cols: lane (col, seg) keeps rows 16 seg .. 16 seg + 15 of value channel col.
+// ag [T][H D + H V]: the decay's and the gate's second products; a_log [H], dt_bias [H D] float.
+template <int NSEG>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                                                         const float* __restrict__ vc, const float* __restrict__ beta,
+                                                         const float* __restrict__ ag, const float* __restrict__ a_log,
+                                                         const float* __restrict__ dt_bias,
+                                                         const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
+                                                         float* __restrict__ state, int64_t state_stride, DeltaDims dm,
+                                                         int cols, int col_blocks, float* __restrict__ o_raw) {
+  constexpr int DP = DR_ROWS * NSEG;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* qs = lds;                          // [DR_CHUNK][DP]
+  float* ks = qs + DR_CHUNK * DP;
+  float* gs = ks + DR_CHUNK * DP;
+  float* vs = gs + DR_CHUNK * DP;           // [DR_CHUNK][cols]
+  float* bs = vs + DR_CHUNK * cols;         // [DR_CHUNK]
+  const int H = dm.H, G = dm.G, D = dm.D, V = dm.V;
+  const int h = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks, b = blockIdx.y;
+  const int gq = h / (H / G);
+  const int tid = threadIdx.x, seg = tid % NSEG, cl = tid / NSEG;
+  const int col = cb * cols + cl;
+  const bool col_ok = cl < cols && col < V;
+  const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0;
+  float* S = state + (size_t)slots[b] * state_stride + (size_t)h * D * V;
+  float s[DR_ROWS];
+#pragma unroll
+  for (int i = 0; i < DR_ROWS; ++i) {
+    const int r = seg * DR_ROWS + i;
+    s[i] = col_ok && r < D ? S[(size_t)r * V + col] : 0.f;
+  }
+  const float rate = expf(a_log[h]);
+  const int AGW = H * D + H * V;
+  for (int c0 = 0; c0 < n; c0 += DR_CHUNK) {
+    const int nc = min(DR_CHUNK, n - c0);
+    __syncthreads();
+    for (int idx = tid; idx < nc * DP; idx += blockDim.x) {
+      const int c = idx / DP, r = idx % DP;
+      const size_t t = (size_t)(t0 + c0 + c);
+      float q = 0.f, k = 0.f, g = 1.f;
+      if (r < D) {
+        q = qn[t * G * D + (size_t)gq * D + r];
+        k = kn[t * G * D + (size_t)gq * D + r];
+        g = expf(-rate * softplus_f(ag[t * AGW + (size_t)h * D + r] + dt_bias[h * D + r]));
+      }
+      qs[idx] = q;
+      ks[idx] = k;
+      gs[idx] = g;
+    }
+    for (int idx = tid; idx < nc * cols; idx += blockDim.x) {
+      const int c = idx / cols, j = cb * cols + idx % cols;
+      vs[idx] = j < V ? vc[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + j] : 0.f;
+    }
+    if (tid < nc) bs[tid] = beta[(size_t)(t0 + c0 + tid) * H + h];
+    __syncthreads();
+    for (int c = 0; c < nc; ++c) {
+      const float* qr = qs + c * DP + seg * DR_ROWS;
+      const float* kr = ks + c * DP + seg * DR_ROWS;
+      const float* gr = gs + c * DP + seg * DR_ROWS;
+      float kk[DR_ROWS];
+      float d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DR_ROWS; ++i) {
+        kk[i] = kr[i];
+        const float q = qr[i];
+        s[i] *= gr[i];
+        d1 = fmaf(s[i], kk[i], d1);
+        d2 = fmaf(s[i], q, d2);
+        d3 = fmaf(kk[i], q, d3);
+      }
+#pragma unroll
+      for (int o = NSEG / 2; o > 0; o >>= 1) {
+        d1 += __shfl_xor(d1, o, TQ_WAVE);
+        d2 += __shfl_xor(d2, o, TQ_WAVE);
+        d3 += __shfl_xor(d3, o, TQ_WAVE);
+      }
+      const float u = bs[c] * (vs[c * cols + (cl < cols ? cl : 0)] - d1);
+#pragma unroll
+      for (int i = 0; i < DR_ROWS; ++i) s[i] = fmaf(kk[i], u, s[i]);
+      // the read-out of the state that holds this token's write: (g S)^T q + u (k . q)
+      if (col_ok && seg == 0) o_raw[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + col] = fmaf(u, d3, d2);
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < DR_ROWS; ++i) {
+      const int r = seg * DR_ROWS + i;
+      if (r < D) S[(size_t)r * V + col] = s[i];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ norm, gate, new inputs
+// grid (T + B), block 256.  Blocks 0 .. T - 1: a wave per head of its token: o / rms(o) * w * sigmoid(gate).
+// Blocks T ..: the convolution's state of one sequence: its last taps - 1 inputs, those of this run and, where the run
+// is shorter, the most recent of the old state before them.
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const float* __restrict__ ag,
+                                                        const float* __restrict__ norm_w, float eps,
+                                                        const float* __restrict__ P, const int* __restrict__ cu_seqlens,
+                                                        const int* __restrict__ slots, float* __restrict__ state,
+                                                        int64_t state_stride, DeltaDims dm, int T,
+                                                        act_t* __restrict__ out) {
+  const int H = dm.H, D = dm.D, V = dm.V, K = dm.taps;
+  if ((int)blockIdx.x < T) {
+    const int t = blockIdx.x, wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+    const int AGW = H * D + H * V;
+    for (int h = wave; h < H; h += 4) {
+      const float* o = o_raw + (size_t)t * H * V + (size_t)h * V;
+      float ss = 0.f;
+      for (int j = lane; j < V; j += TQ_WAVE) ss += o[j] * o[j];
+      ss = wave_sum(ss);
+      const float rs = 1.0f / sqrtf(ss / (float)V + eps);
+      const float* gate = ag + (size_t)t * AGW + (size_t)H * D + (size_t)h * V;
+      for (int j = lane; j < V; j += TQ_WAVE)
+        out[(size_t)t * H * V + (size_t)h * V + j] = from_f32<act_t>(o[j] * rs * norm_w[j] * sigmoid_f(gate[j]));
+    }
+    return;
+  }
+  const int b = blockIdx.x - T;
+  const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0;
+  const int C = dd_channels(dm), NP = dd_np(dm);
+  float* hist = state + (size_t)slots[b] * state_stride + (size_t)H * D * V;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float* hc = hist + (size_t)c * (K - 1);
+    // new[m], m = 0 .. K - 2 oldest first, is the input K - 1 - m tokens before the run's end
+    for (int m = 0; m < K - 1; ++m) {
+      const int back = K - 1 - m;           // 1 = the run's last token
+      // ascending m reads old entries at m + n >= m: none that this loop has already overwritten
+      hc[m] = back <= n ? P[(size_t)(t0 + n - back) * NP + c] : hc[m + n];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ entry points
+static int dims_ok(const DeltaDims& d) {
+  return d.H > 0 && d.G > 0 && d.H % d.G == 0 && d.D > 0 && d.D <= 256 && d.V > 0 && d.taps >= 1 && d.taps <= 64 &&
+         d.ra > 0 && d.rg > 0;
+}
+
+// Floats of one sequence's row of state.
+TQ_API int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps) {
+  const DeltaDims d{H, G, D, V, taps, 1, 1};
+  return dd_state(d);
+}
+
+// P [T][NP] float (see the head of this file); slot_of_token [T]; state: rows of state_stride floats by slot;
+// conv_w [channels][taps] float.  Writes qn, kn [T][G D], vc [T][H V], beta [T][H] (float) and low [T][ra + rg]
+// (activation type).
+TQ_API int tq_delta_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
+                         const float* conv_w, int H, int G, int D, int V, int taps, int ra, int rg, float* qn, float* kn,
+                         float* vc, float* beta, void* low, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  const DeltaDims d{H, G, D, V, taps, ra, rg};
+  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(T), dim3(256), 0, st, P, slot_of_token, state, state_stride, conv_w, d, qn,
+                     kn, vc, beta, (act_t*)low);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// The recurrence over runs of tokens, one run per sequence (cu_seqlens [B + 1], slots [B]); the state rows are read
+// and written.  o_raw [T][H V] float.
+TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, const float* ag,
+                         const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
+                         int64_t state_stride, int H, int G, int D, int V, int taps, int B, float* o_raw,
+                         hipStream_t st) {
+  if (B <= 0) return 0;
+  const DeltaDims d{H, G, D, V, taps, 1, 1};
+  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
+  if (B > 65535) return TQ_ERR_UNSUPPORTED;
+  int nseg = 1;
+  while (nseg * DR_ROWS < D) nseg *= 2;
+  const int cols = V < 256 / nseg ? V : 256 / nseg;
+  const int col_blocks = (V + cols - 1) / cols;
+  // whole waves, so that the lanes of a value channel always lie in one
+  const int threads = (nseg * cols + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
+  const size_t shmem = ((size_t)3 * DR_CHUNK * DR_ROWS * nseg + (size_t)DR_CHUNK * cols + DR_CHUNK) * sizeof(float);
+#define TQ_SCAN(NS)                                                                                                   \
+  if (shmem > 48 * 1024)                                                                                              \
+    (void)hipFuncSetAttribute((const void*)delta_scan_kernel<NS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
+  hipLaunchKernelGGL(delta_scan_kernel<NS>, dim3(H * col_blocks, B), dim3(threads), shmem, st, qn, kn, vc, beta, ag,   \
+                     a_log, dt_bias, cu_seqlens, slots, state, state_stride, d, cols, col_blocks, o_raw)
+  switch (nseg) {
+    case 1: TQ_SCAN(1); break;
+    case 2: TQ_SCAN(2); break;
+    case 4: TQ_SCAN(4); break;
+    case 8: TQ_SCAN(8); break;
+    default: TQ_SCAN(16); break;
+  }
+#undef TQ_SCAN
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// Norm and gate of every head's read-out into `out` [T][H V] (activation type), and every sequence's new convolution
+// state from P.  norm_w [V] float.
+TQ_API int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w, float eps, const float* P,
+                        const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
+                        int V, int taps, int ra, int rg, int T, int B, void* out, hipStream_t st) {
+  if (T <= 0 || B <= 0) return 0;
+  const DeltaDims d{H, G, D, V, taps, ra, rg};
+  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(delta_out_kernel, dim3(T + B), dim3(256), 0, st, o_raw, ag, norm_w, eps, P, cu_seqlens, slots, state,
+                     state_stride, d, T, (act_t*)out);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}

@@ -523,3 +523,166 @@ TQ_API int tq_moe_combine(const float* y, const int* pair_slot, const float* wei
   TQ_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------- embedding with a learned position row
+// x[t, :] = table[tokens[t], :] * scale + pos_table[positions[t], :], in float: for models that add a learned vector
+// per position to the embedded token instead of rotating queries and keys.
+template <class W>
+__global__ void embed_pos_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                                 const W* __restrict__ table, const W* __restrict__ pos_table, float* __restrict__ x,
+                                 int H, float scale) {
+  const int t = blockIdx.x;
+  const W* row = table + (size_t)tokens[t] * H;
+  const W* prow = pos_table + (size_t)positions[t] * H;
+  float* out = x + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32(row[i]) * scale + to_f32(prow[i]);
+}
+
+TQ_API int tq_embed_pos(const int* tokens, const int* positions, const void* table, const void* pos_table, int wtype,
+                        float* x, int T, int H, float scale, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (!positions || !pos_table) return TQ_ERR_BAD_ARG;
+  TQ_DISPATCH_W(wtype, {
+    hipLaunchKernelGGL(embed_pos_kernel<W>, dim3(T), dim3(256), 0, st, tokens, positions, (const W*)table,
+                       (const W*)pos_table, x, H, scale);
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- residual sum of a normed part + RMS norm
+// For layers that norm a part's output before it joins the stream (a norm before and one after every part):
+//   d = what add_rmsnorm would add (partial sums in order, or the experts' weighted rows and the gated dense sums)
+//   v = x[row] + (d * (1 / sqrt(mean(d^2) + eps_d))) * wd          (the residual sum, in float)
+//   x[row] = v                                                       (only when rows is null)
+//   out = (v * (1 / sqrt(mean(v^2) + eps))) * w                      (left out when w is null)
+// Both sums of squares run in the fixed order of block_sum over a thread's own elements, whatever the step holds.
+template <class W, bool VEC>
+__global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta, int S,
+                                          size_t delta_stride, const float* __restrict__ y,
+                                          const int* __restrict__ pair_slot, const float* __restrict__ weights,
+                                          int topk, const float* __restrict__ gate, const W* __restrict__ wd,
+                                          float eps_d, const W* __restrict__ w, float eps,
+                                          const int* __restrict__ rows, act_t* __restrict__ out,
+                                          float* __restrict__ out32, int H) {
+  extern __shared__ __attribute__((aligned(16))) float v[];       // H floats, then one float per wave
+  __shared__ int slot[64];
+  __shared__ float wgt[64];
+  float* red = v + (H + 3) / 4 * 4;
+  const int r = blockIdx.x;
+  const int row = rows ? rows[r] : r;
+  float* xr = x + (size_t)row * H;
+  const float* dr = delta + (size_t)row * H;
+  float g = 1.0f;
+  if (y) {
+    if (threadIdx.x < topk) {
+      slot[threadIdx.x] = pair_slot[(size_t)row * topk + threadIdx.x];
+      wgt[threadIdx.x] = weights[(size_t)row * topk + threadIdx.x];
+    }
+    if (gate) g = gate[row];
+    __syncthreads();
+  }
+  constexpr int N = VEC ? 4 : 1;
+  float ss = 0.f;
+  for (int i = threadIdx.x * N; i < H; i += blockDim.x * N) {
+    float d[N];
+#pragma unroll
+    for (int u = 0; u < N; ++u) d[u] = 0.f;
+    if (y) {
+      for (int j = 0; j < topk; ++j) {
+        const float* yr = y + (size_t)slot[j] * H + i;
+        if constexpr (VEC) {
+          const f32x4 t = load4f(yr);
+          d[0] += wgt[j] * t.x;
+          d[1] += wgt[j] * t.y;
+          d[2] += wgt[j] * t.z;
+          d[3] += wgt[j] * t.w;
+        } else {
+          d[0] += wgt[j] * yr[0];
+        }
+      }
+      if (S > 0) {
+        float sh[N];
+#pragma unroll
+        for (int u = 0; u < N; ++u) sh[u] = 0.f;
+        for (int s = 0; s < S; ++s)
+#pragma unroll
+          for (int u = 0; u < N; ++u) sh[u] += dr[s * delta_stride + i + u];
+#pragma unroll
+        for (int u = 0; u < N; ++u) d[u] += g * sh[u];
+      }
+    } else {
+      for (int s = 0; s < S; ++s) {
+        if constexpr (VEC) {
+          const f32x4 t = load4f(dr + s * delta_stride + i);
+          d[0] += t.x;
+          d[1] += t.y;
+          d[2] += t.z;
+          d[3] += t.w;
+        } else {
+          d[0] += dr[s * delta_stride + i];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      v[i + u] = d[u];
+      ss += d[u] * d[u];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rd = 1.0f / sqrtf(ss / (float)H + eps_d);
+  float s2 = 0.f;
+  for (int i = threadIdx.x * N; i < H; i += blockDim.x * N) {
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      const float a = xr[i + u] + (v[i + u] * rd) * to_f32(wd[i + u]);
+      v[i + u] = a;
+      if (!rows) xr[i + u] = a;
+      s2 += a * a;
+    }
+  }
+  if (!w) return;
+  s2 = block_sum(s2, red);
+  const float rs = 1.0f / sqrtf(s2 / (float)H + eps);
+  for (int i = threadIdx.x * N; i < H; i += blockDim.x * N) {
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      const float o = v[i + u] * rs * to_f32(w[i + u]);
+      if (out) out[(size_t)r * H + i + u] = from_f32<act_t>(o);
+      if (out32) out32[(size_t)r * H + i + u] = o;
+    }
+  }
+}
+
+// As tq_add_rmsnorm, with the weights wd and the eps_d of the norm that what is added passes first; w null: the
+// stream is summed and nothing is normed (no out, no out32).
+TQ_API int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
+                                 const int* pair_slot, const float* weights, int topk, const float* gate,
+                                 const void* wd, float eps_d, const void* w, int wtype, float eps, const int* rows,
+                                 int R, void* out, float* out32, int H, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (!wd || (y && (topk < 1 || topk > 64 || !pair_slot || !weights))) return TQ_ERR_BAD_ARG;
+  if (!y && (S < 1 || !delta)) return TQ_ERR_BAD_ARG;
+  const int threads = (H % 4 == 0 && H >= 2048) ? 512 : 256;
+  const size_t shmem = (size_t)((H + 3) / 4 * 4 + threads / TQ_WAVE) * sizeof(float);
+  if (shmem > 150 * 1024) return TQ_ERR_UNSUPPORTED;
+  const bool vec = H % 4 == 0;
+  TQ_DISPATCH_W(wtype, {
+    if (vec) {
+      if (shmem > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)add_normed_rmsnorm_kernel<W, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+      hipLaunchKernelGGL((add_normed_rmsnorm_kernel<W, true>), dim3(R), dim3(threads), shmem, st, x, delta, S,
+                         (size_t)delta_stride, y, pair_slot, weights, topk, gate, (const W*)wd, eps_d, (const W*)w, eps,
+                         rows, (act_t*)out, out32, H);
+    } else {
+      if (shmem > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)add_normed_rmsnorm_kernel<W, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+      hipLaunchKernelGGL((add_normed_rmsnorm_kernel<W, false>), dim3(R), dim3(threads), shmem, st, x, delta, S,
+                         (size_t)delta_stride, y, pair_slot, weights, topk, gate, (const W*)wd, eps_d, (const W*)w, eps,
+                         rows, (act_t*)out, out32, H);
+    }
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}

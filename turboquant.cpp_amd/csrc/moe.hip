@@ -139,8 +139,12 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
 
 // One wave chooses for one token.  src: the token's `rows` logits; lg: E floats of LDS for this wave; ids,
 // weights, shared_gate: where the token's results go; ids2: a second place for the ids (LDS), or null.
+// groups > 1: the experts form `groups` equal groups of neighbours; a group's score is its largest logit (the order of
+// softmax scores is the order of logits), only experts of the `keep` best groups can be chosen (among groups of
+// equal score the highest index wins, as among experts), and the softmax over all experts is taken before the
+// others are left out.
 __device__ __forceinline__ void select_token(const float* __restrict__ src, int rows, int E, int topk, int renorm,
-                                             float* lg, int* __restrict__ ids, int* ids2,
+                                             int groups, int keep, float* lg, int* __restrict__ ids, int* ids2,
                                              float* __restrict__ weights, float* __restrict__ shared_gate) {
   const int lane = threadIdx.x % TQ_WAVE;
   for (int e = lane; e < E; e += TQ_WAVE) lg[e] = src[e];
@@ -154,6 +158,50 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
     float d = 0.f;
     for (int e = lane; e < E; e += TQ_WAVE) d += expf(lg[e] - mx);
     denom = wave_sum(d);
+  }
+  if (groups > 1 && keep < groups) {
+    const int per = E / groups;
+    // a lane per group (in turns of 64): the group's largest logit; then `keep` rounds choose the best groups
+    float gmax[4];      // up to 256 groups
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int gi = lane + 64 * i;
+      float m = -INFINITY;
+      if (gi < groups)
+        for (int e = gi * per; e < (gi + 1) * per; ++e) m = fmaxf(m, lg[e]);
+      gmax[i] = m;
+    }
+    unsigned kept = 0;      // bit i: group lane + 64 i is kept
+    for (int k = 0; k < keep; ++k) {
+      float bv = -INFINITY;
+      int bi = -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int gi = lane + 64 * i;
+        if (gi < groups && !((kept >> i) & 1u) && gmax[i] >= bv) {
+          bv = gmax[i];
+          bi = gi;
+        }
+      }
+#pragma unroll
+      for (int o = TQ_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, TQ_WAVE);
+        const int oi = __shfl_xor(bi, o, TQ_WAVE);
+        if (oi >= 0 && (bi < 0 || ov > bv || (ov == bv && oi > bi))) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (bi >= 0 && bi % 64 == lane) kept |= 1u << (bi / 64);
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int gi = lane + 64 * i;
+      if (gi < groups && !((kept >> i) & 1u))
+        for (int e = gi * per; e < (gi + 1) * per; ++e) lg[e] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
   }
   float sel = 0.f;    // lane k keeps the k-th selected logit
   for (int k = 0; k < topk; ++k) {
@@ -195,14 +243,14 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
 }
 
 __global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int rows, int E,
-                                                            int topk, int renorm, int* __restrict__ ids,
-                                                            float* __restrict__ weights,
+                                                            int topk, int renorm, int groups, int keep,
+                                                            int* __restrict__ ids, float* __restrict__ weights,
                                                             float* __restrict__ shared_gate, int T) {
   extern __shared__ float sm[];      // [4][E]
   const int wave = threadIdx.x / TQ_WAVE;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
-  select_token(logits + (size_t)t * rows, rows, E, topk, renorm, sm + wave * E, ids + (size_t)t * topk, nullptr,
+  select_token(logits + (size_t)t * rows, rows, E, topk, renorm, groups, keep, sm + wave * E, ids + (size_t)t * topk, nullptr,
                weights + (size_t)t * topk, shared_gate + t);
 }
 
@@ -248,18 +296,31 @@ static int launch_router_logits(const float* x, const void* wr, const void* shar
 }
 
 // logits: scratch of T * (E + 1) floats (T * E without a shared gate vector).
-TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
-                          int renorm, int* ids, float* weights, float* shared_gate, float* logits, int T, int H,
-                          hipStream_t st) {
+// Whether a choice within the best `keep` of `groups` groups of experts can be made: groups == 1 means none.
+static int groups_ok(int E, int topk, int groups, int keep) {
+  if (groups == 1) return 1;
+  return groups >= 1 && groups <= 256 && E % groups == 0 && keep >= 1 && keep <= groups && topk <= keep * (E / groups);
+}
+
+TQ_API int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
+                                  int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                                  float* logits, int T, int H, hipStream_t st) {
   if (T <= 0) return 0;
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
+  if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
   const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
   if (rc) return rc;
   const int rows = E + (shared_w ? 1 : 0);
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
-                     rows, E, topk, renorm, ids, weights, shared_gate, T);
+                     rows, E, topk, renorm, groups, keep, ids, weights, shared_gate, T);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
+                          int renorm, int* ids, float* weights, float* shared_gate, float* logits, int T, int H,
+                          hipStream_t st) {
+  return tq_router_topk_grouped(x, wr, shared_w, wtype, E, topk, renorm, 1, 1, ids, weights, shared_gate, logits, T, H, st);
 }
 
 // ---------------------------------------------------------------- order of pairs by expert
@@ -553,8 +614,8 @@ static int launch_align_multi(const int* ids, int n_pairs, int E, int topk, int 
 // then all waves order the pairs; the same device functions and so the same results as the two kernels.
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __restrict__ logits, int rows, int E,
-                                                               int topk, int renorm, int* __restrict__ ids,
-                                                               float* __restrict__ weights,
+                                                               int topk, int renorm, int groups, int keep,
+                                                               int* __restrict__ ids, float* __restrict__ weights,
                                                                float* __restrict__ shared_gate, int T, int unit,
                                                                int cap, int* __restrict__ sorted_token,
                                                                int* __restrict__ pair_slot,
@@ -566,7 +627,7 @@ __global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __re
   float* lg = (float*)(ids_l + NW * topk);
   const int wave = threadIdx.x / TQ_WAVE;
   if (wave < T)
-    select_token(logits + (size_t)wave * rows, rows, E, topk, renorm, lg + wave * E, ids + (size_t)wave * topk,
+    select_token(logits + (size_t)wave * rows, rows, E, topk, renorm, groups, keep, lg + wave * E, ids + (size_t)wave * topk,
                  ids_l + wave * topk, weights + (size_t)wave * topk, shared_gate + wave);
   __syncthreads();
   align_pairs<NW>(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
@@ -591,13 +652,17 @@ TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, 
 // tq_router_topk followed by tq_moe_align; up to 16 tokens take two kernels instead of three, and from 8,192 pairs on
 // several workgroups order the pairs (the same order).  logits: scratch of T * (E + 1) floats (T * E without a shared
 // gate vector); what it holds afterwards means nothing.
-TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
-                    int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap, int* sorted_token,
-                    int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st) {
+// groups, keep: the choice within the best `keep` of `groups` groups of experts (1, 1: among all).
+TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+                            int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int unit,
+                            int cap, int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H,
+                            hipStream_t st) {
   if (T <= 0) return 0;
+  if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
   const size_t shmem = ((size_t)(AW + 1) * E + (size_t)AW * topk + (size_t)AW * E) * 4;
   if (T > AW || shmem > 64 * 1024) {
-    const int rc = tq_router_topk(x, wr, shared_w, wtype, E, topk, renorm, ids, weights, shared_gate, logits, T, H, st);
+    const int rc = tq_router_topk_grouped(x, wr, shared_w, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate,
+                                          logits, T, H, st);
     if (rc) return rc;
     // once the experts are chosen the logits are done with: the order by several workgroups keeps its table there
     const int n = T * topk;
@@ -615,14 +680,21 @@ TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wt
   if (T == 1) {      // one wave: its barriers cost nothing
     const size_t shmem1 = ((size_t)2 * E + topk + E) * 4;
     hipLaunchKernelGGL(select_align_kernel<1>, dim3(1), dim3(64), shmem1, st, logits, E + (shared_w ? 1 : 0), E, topk,
-                       renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
+                       renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
     TQ_LAUNCH_CHECK();
     return 0;
   }
   if (shmem > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)select_align_kernel<AW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(select_align_kernel<AW>, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
-                     renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
+                     renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+                    int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap, int* sorted_token,
+                    int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st) {
+  return tq_route_grouped(x, wr, shared_w, wtype, E, topk, renorm, 1, 1, ids, weights, shared_gate, logits, unit, cap,
+                          sorted_token, pair_slot, tile_expert, n_tiles, T, H, st);
 }

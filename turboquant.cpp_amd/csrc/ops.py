@@ -57,6 +57,22 @@ _SIGNATURES = {
     "tq_probs_half": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
     "tq_sample_topp_scratch": [_c_int],
+    "tq_embed_pos": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
+    "tq_add_normed_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr,
+                              _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_attention_generic_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
+                                 _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
+    "tq_router_topk_grouped": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                               _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_route_grouped": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                         _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_delta_state_floats": [_c_int, _c_int, _c_int, _c_int, _c_int],
+    "tq_delta_prep": [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                      _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_delta_scan": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int,
+                      _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_delta_out": [_c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 # entry points that only one of the two libraries has
@@ -77,6 +93,12 @@ _OPTIONAL = {
     "tq_probe_stream": [_c_ptr, _c_i64, _c_int, ctypes.c_uint, _c_ptr, _c_ptr],
     "tq_probe_mfma": [_c_int, _c_int, _c_int, ctypes.c_uint, _c_ptr, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
+    "tq_attention_f32_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                             _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
+                             _c_int, _c_ptr],
+    "tq_attention_mfma_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                              _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
+                              _c_int, _c_ptr],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
@@ -116,6 +138,7 @@ def library(dtype) -> ctypes.CDLL:
             f = getattr(lib, fn)
             f.argtypes, f.restype = sig, _c_int
     lib.tq_sample_topp_scratch.restype = _c_i64
+    lib.tq_delta_state_floats.restype = _c_i64
     for fn in ("tq_attention_decode_scratch", "tq_attention_f32_scratch"):
         if hasattr(lib, fn):
             getattr(lib, fn).restype = _c_i64
@@ -163,7 +186,8 @@ def _check(t: torch.Tensor, kernel: str, name: str, dtype=None, shape=None) -> N
 _PROFILE: list | None = None
 _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pair": "matmul", "qkv_rope_write": "matmul",
          "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
-         "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe"}
+         "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
+         "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn"}
 
 
 def profile_begin() -> None:
@@ -212,14 +236,23 @@ def _run(kernel: str, code: int, kind: str | None = None) -> None:
 
 
 # ------------------------------------------------------------------ row-wise kernels
-def embed(tokens: torch.Tensor, table: torch.Tensor, act, scale: float = 1.0) -> torch.Tensor:
-    """x[t] = table[tokens[t]] (times ``scale``) as float32 [T, H]."""
+def embed(tokens: torch.Tensor, table: torch.Tensor, act, scale: float = 1.0, pos_table: torch.Tensor | None = None,
+          positions: torch.Tensor | None = None) -> torch.Tensor:
+    """x[t] = table[tokens[t]] (times ``scale``) as float32 [T, H]; with ``pos_table`` [P, H] and ``positions`` [T],
+    plus pos_table[positions[t]] (a learned vector per position; positions beyond the table are the caller's to refuse)."""
     k = "embed"
     _check(tokens, k, "tokens", torch.int32)
     _need(tokens.dim() == 1 and table.dim() == 2, k, "tokens [T], table [V, H]")
     _check(table, k, "table", tuple(_WTYPE))
     T, (V, H) = tokens.numel(), table.shape
     x = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    if pos_table is not None:
+        _check(pos_table, k, "pos_table", table.dtype)
+        _need(pos_table.dim() == 2 and pos_table.shape[1] == H, k, lambda: f"pos_table must be [P, {H}]")
+        _check(positions, k, "positions", torch.int32, (T,))
+        _run(k, library(act).tq_embed_pos(_ptr(tokens), _ptr(positions), _ptr(table), _ptr(pos_table), _WTYPE[table.dtype],
+                                          _ptr(x), T, H, float(scale), _stream()))
+        return x
     _run(k, library(act).tq_embed(_ptr(tokens), _ptr(table), _WTYPE[table.dtype], _ptr(x), T, H, float(scale), _stream()))
     return x
 
@@ -272,16 +305,44 @@ class GatheredSum:
         return moe_combine(self.y, self.pair_slot, self.weights, self.dense, self.gate, act)
 
 
-def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
+@dataclasses.dataclass
+class NormedDelta:
+    """A part's output that joins the residual stream only after an RMS norm of its own:
+    ``x += rmsnorm(inner, eps) * weight``, ``inner`` being float32 partial sums [S, T, H] or a GatheredSum.  The next
+    norm does both in one pass; ``materialize`` gives the normed tensor [1, T, H] to whoever needs it earlier."""
+    inner: object
+    weight: torch.Tensor
+    eps: float
+
+    def materialize(self, act) -> torch.Tensor:
+        ref = self.inner.y if isinstance(self.inner, GatheredSum) else self.inner
+        T = self.inner.pair_slot.shape[0] if isinstance(self.inner, GatheredSum) else ref.shape[1]
+        x = torch.zeros((T, ref.shape[-1]), dtype=torch.float32, device=ref.device)
+        add_rmsnorm(x, self, None, 0.0, act, want_act=False)
+        return x[None]
+
+
+def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float, act,
                 rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False):
     """x += delta (in place, unless ``rows`` picks rows), where delta is None, float32 partial sums [S, T, H] added
-    one after the other, or a GatheredSum; returns rmsnorm(x) * weight as (activation-typed or None, float32 or
-    None), one row per entry of ``rows`` (all rows if None)."""
+    one after the other, a GatheredSum, or a NormedDelta around either (then what is added is its RMS norm); returns
+    rmsnorm(x) * weight as (activation-typed or None, float32 or None), one row per entry of ``rows`` (all rows if
+    None).  ``weight`` None (with a NormedDelta only): the stream is summed and nothing is returned."""
     k = "add_rmsnorm"
     _check(x, k, "x", torch.float32)
     _need(x.dim() == 2, k, "x must be [T, H]")
     T, H = x.shape
-    _check(weight, k, "weight", tuple(_WTYPE), (H,))
+    post = None
+    if isinstance(delta, NormedDelta):
+        post, delta = delta, delta.inner
+        _check(post.weight, k, "the added part's norm weight", tuple(_WTYPE), (H,))
+        _need(delta is not None, k, "a normed part needs something to norm")
+    if weight is None:
+        _need(post is not None and rows is None, k, "without a weight only a normed part can be summed, into all rows")
+        want_act = want_f32 = False
+    else:
+        _check(weight, k, "weight", tuple(_WTYPE), (H,))
+        _need(post is None or post.weight.dtype == weight.dtype, k, "the two norms' weights must have one type")
     y = pair_slot = weights = gate = None
     topk = 0
     if isinstance(delta, GatheredSum):
@@ -308,6 +369,12 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
     adt = ACT_DTYPES[dtype_name(act)]
     out = torch.empty((R, H), dtype=adt, device=x.device) if want_act else None
     out32 = torch.empty((R, H), dtype=torch.float32, device=x.device) if want_f32 else None
+    if post is not None:
+        _run(k, library(act).tq_add_normed_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights),
+                                                   topk, _ptr(gate), _ptr(post.weight), float(post.eps), _ptr(weight),
+                                                   _WTYPE[post.weight.dtype], float(eps), _ptr(rows), R, _ptr(out),
+                                                   _ptr(out32), H, _stream()))
+        return out, out32
     _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights), topk,
                                         _ptr(gate), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(rows), R,
                                         _ptr(out), _ptr(out32), H, _stream()))
@@ -754,8 +821,13 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
 def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, layer_offset: int,
               positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, page_size: int,
               page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-              scale: float, act, runs: dict | None = None) -> torch.Tensor:
+              scale: float, act, runs: dict | None = None, softcap: float | None = None,
+              distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None) -> torch.Tensor:
     """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
+
+    ``softcap`` c: a scaled score s becomes c tanh(s / c).  ``distance_bias`` (r1, r2), float32 [nh] each: then
+    r1[h] ln(1 + r2[h] (i - j)) is taken off the score of query position i and key position j.  ``chunk`` n: position i
+    sees j only if i // n == j // n, beside j <= i and the window.
 
     ``seq_of_token`` gives each token's row of ``block_table`` (its slot).  ``runs`` describes the same tokens
     as runs of consecutive positions, one per sequence, for the kernels that work on tiles of tokens:
@@ -777,6 +849,14 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     out = torch.empty_like(q)
     esz = k_pages.element_size()
     lib = library(act)
+    cap = float(softcap or 0.0)
+    _need(cap >= 0 and (chunk is None or chunk >= 1), k, "softcap and chunk must be positive")
+    r1 = r2 = None
+    if distance_bias is not None:
+        r1, r2 = distance_bias
+        _check(r1, k, "r1", torch.float32, (num_heads,))
+        _check(r2, k, "r2", torch.float32, (num_heads,))
+    mod = (cap, _ptr(r1), _ptr(r2), int(chunk or 0))
     if (runs is not None and dtype_name(act) == "bfloat16" and hasattr(lib, "tq_attention_mfma")
             and head_dim % 16 == 0 and head_dim <= 256 and page_size % 64 == 0 and page_stride % 8 == 0 and scale > 0):
         B = runs["slots"].numel()
@@ -789,10 +869,10 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_mfma", lib.tq_attention_mfma(
+        _run("attention_mfma", lib.tq_attention_mfma_mod(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
-            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), _ptr(out),
+            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
         return out
     if (runs is not None and dtype_name(act) == "float32" and hasattr(lib, "tq_attention_f32") and head_dim % 4 == 0
@@ -807,29 +887,41 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_f32_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_f32", lib.tq_attention_f32(
+        _run("attention_f32", lib.tq_attention_f32_mod(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
-            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), _ptr(out),
+            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
         return out
-    _run(k, lib.tq_attention_generic(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
-                                              v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
-                                              _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
-                                              page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),
-                                              float(scale), _ptr(out), _stream()))
+    _run(k, lib.tq_attention_generic_mod(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
+                                         v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
+                                         _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
+                                         page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),
+                                         float(scale), *mod, _ptr(out), _stream()))
     return out
 
 
 # ------------------------------------------------------------------ routing
+def _expert_groups(k: str, E: int, top_k: int, groups) -> tuple[int, int]:
+    """(count, keep) of a choice within the best ``keep`` of ``count`` equal groups of neighbouring experts."""
+    if groups is None:
+        return 1, 1
+    count, keep = int(groups[0]), int(groups[1])
+    _need(1 <= count <= 256 and E % count == 0 and 1 <= keep <= count and top_k <= keep * (E // count), k,
+          lambda: f"{count} groups of which {keep} are kept do not fit {E} experts with {top_k} per token")
+    return count, keep
+
+
 def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int,
-                renormalize: bool, act):
-    """ids int32 [T, k], weights float32 [T, k], and sigmoid(x . shared_scale) float32 [T] (or None)."""
+                renormalize: bool, act, groups: tuple[int, int] | None = None):
+    """ids int32 [T, k], weights float32 [T, k], and sigmoid(x . shared_scale) float32 [T] (or None).
+    ``groups`` (count, keep): only experts of the ``keep`` groups with the largest best score can be chosen."""
     k = "router_topk"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
-    _run(k, library(act).tq_router_topk(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits),
-                                        T, H, _stream()))
+    count, keep = _expert_groups(k, E, top_k, groups)
+    _run(k, library(act).tq_router_topk_grouped(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
+                                                int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
+                                                _ptr(logits), T, H, _stream()))
     return ids, weights, gate
 
 
@@ -864,16 +956,18 @@ def _align_outputs(T: int, topk: int, num_experts: int, unit: int, dev):
 
 
 def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int, renormalize: bool,
-          unit: int, act):
+          unit: int, act, groups: tuple[int, int] | None = None):
     """``router_topk`` followed by ``moe_align`` in one call: (ids, weights, gate, sorted_token, pair_slot,
     tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
     k = "route"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
     _need(unit in (16, 32, 64, 128, 256), k, "unit must be 16, 32, 64, 128 or 256")
+    count, keep = _expert_groups(k, E, top_k, groups)
     cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
-    _run(k, library(act).tq_route(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                  int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits), unit, cap,
-                                  _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), T, H, _stream()))
+    _run(k, library(act).tq_route_grouped(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
+                                          int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
+                                          _ptr(logits), unit, cap, _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert),
+                                          _ptr(n_tiles), T, H, _stream()))
     return ids, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles
 
 
@@ -888,6 +982,115 @@ def moe_align(ids: torch.Tensor, num_experts: int, unit: int, act):
     _run(k, library(act).tq_moe_align(_ptr(ids), n_pairs, num_experts, topk, unit, cap, _ptr(sorted_token),
                                       _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), _stream()))
     return sorted_token, pair_slot, tile_expert, n_tiles
+
+
+# ------------------------------------------------------------------ the gated delta rule
+@dataclasses.dataclass(frozen=True)
+class DeltaDims:
+    """Sizes of a delta-rule mixer: heads, q/k heads, key width, value width, convolution taps, and the ranks of the
+    decay's and the gate's first products."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    taps: int
+    rank_a: int
+    rank_g: int
+
+    @property
+    def channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @property
+    def projections(self) -> int:
+        return self.channels + self.heads + self.rank_a + self.rank_g
+
+    @property
+    def state_floats(self) -> int:
+        return self.heads * self.dim * self.vdim + self.channels * (self.taps - 1)
+
+    def sizes(self):
+        return self.heads, self.kv_heads, self.dim, self.vdim, self.taps
+
+
+def _delta_state(k: str, state: torch.Tensor, dims: DeltaDims) -> int:
+    _check(state, k, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] >= dims.state_floats, k,
+          lambda: f"state must be [slots, >= {dims.state_floats}], is {tuple(state.shape)}")
+    _need(dims.heads % dims.kv_heads == 0 and 1 <= dims.dim <= 256 and 1 <= dims.taps <= 64, k,
+          "heads must be a multiple of kv heads, the key width at most 256, the taps at most 64")
+    return state.shape[1]
+
+
+def delta_prep(proj: torch.Tensor, slot_of_token: torch.Tensor, state: torch.Tensor, conv_w: torch.Tensor,
+               dims: DeltaDims, act):
+    """From the float32 projections [T, q | k | v | b | a1 | g1] of a step's tokens: q and k after convolution, silu
+    and scaling to unit length (q also by dim^-1/2) [T, G*dim], v after convolution and silu [T, H*vdim],
+    beta = sigmoid(b) [T, H], all float32, and the low-rank activations [T, rank_a + rank_g] in the activation type.
+    The convolution's inputs before a token's run are read from ``state`` [slots, floats]; nothing is written there."""
+    k = "delta_prep"
+    T = slot_of_token.numel()
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    _check(slot_of_token, k, "slot_of_token", torch.int32, (T,))
+    stride = _delta_state(k, state, dims)
+    _check(conv_w, k, "conv_w", torch.float32, (dims.channels, dims.taps))
+    dev, f32 = proj.device, torch.float32
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    qn = torch.empty((T, G * D), dtype=f32, device=dev)
+    kn = torch.empty((T, G * D), dtype=f32, device=dev)
+    vc = torch.empty((T, H * V), dtype=f32, device=dev)
+    beta = torch.empty((T, H), dtype=f32, device=dev)
+    low = torch.empty((T, dims.rank_a + dims.rank_g), dtype=ACT_DTYPES[dtype_name(act)], device=dev)
+    _run(k, library(act).tq_delta_prep(_ptr(proj), _ptr(slot_of_token), _ptr(state), stride, _ptr(conv_w), *dims.sizes(),
+                                       dims.rank_a, dims.rank_g, _ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(low), T,
+                                       _stream()))
+    return qn, kn, vc, beta, low
+
+
+def delta_scan(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, ag: torch.Tensor,
+               a_log: torch.Tensor, dt_bias: torch.Tensor, runs: dict, state: torch.Tensor, dims: DeltaDims, act):
+    """The recurrence over each sequence's run of tokens, in order, from and into its row of ``state``:
+    S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with g = exp(-exp(a_log) softplus(a + dt_bias))
+    from the first H*dim columns of ``ag`` [T, H*dim + H*vdim].  Returns o, float32 [T, H*vdim]."""
+    k = "delta_scan"
+    T = qn.shape[0]
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    for name, t, w in (("qn", qn, G * D), ("kn", kn, G * D), ("vc", vc, H * V), ("beta", beta, H), ("ag", ag, H * D + H * V)):
+        _check(t, k, name, torch.float32, (T, w))
+    _check(a_log, k, "a_log", torch.float32, (H,))
+    _check(dt_bias, k, "dt_bias", torch.float32, (H * D,))
+    stride = _delta_state(k, state, dims)
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    o = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)
+    _run(k, library(act).tq_delta_scan(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(ag), _ptr(a_log), _ptr(dt_bias),
+                                       _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), B,
+                                       _ptr(o), _stream()))
+    return o
+
+
+def delta_out(o: torch.Tensor, ag: torch.Tensor, norm_w: torch.Tensor, eps: float, proj: torch.Tensor, runs: dict,
+              state: torch.Tensor, dims: DeltaDims, act) -> torch.Tensor:
+    """Every head's read-out divided by its root mean square, times ``norm_w`` [vdim], times the sigmoid of the gate
+    (the last H*vdim columns of ``ag``), in the activation type [T, H*vdim]; and the convolution's part of every
+    sequence's state brought to the end of its run."""
+    k = "delta_out"
+    T = o.shape[0]
+    H, D, V = dims.heads, dims.dim, dims.vdim
+    _check(o, k, "o", torch.float32, (T, H * V))
+    _check(ag, k, "ag", torch.float32, (T, H * D + H * V))
+    _check(norm_w, k, "norm_w", torch.float32, (V,))
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    stride = _delta_state(k, state, dims)
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    out = torch.empty((T, H * V), dtype=ACT_DTYPES[dtype_name(act)], device=o.device)
+    _run(k, library(act).tq_delta_out(_ptr(o), _ptr(ag), _ptr(norm_w), float(eps), _ptr(proj), _ptr(runs["cu_seqlens"]),
+                                      _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), dims.rank_a, dims.rank_g, T,
+                                      B, _ptr(out), _stream()))
+    return out
 
 
 # ------------------------------------------------------------------ sampling

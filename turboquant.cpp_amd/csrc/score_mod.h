@@ -1,0 +1,38 @@
+// What a model may do to an attention score between the product of query and key and the softmax, and which
+// positions a token may see at all.  Every attention kernel takes the same description:
+//
+//   cap > 0        score <- cap * tanh(score / cap), after the scale
+//   r1, r2         (per query head; null: none) then score <- score - r1[h] * ln(1 + r2[h] * (i - j)) for a query at
+//                  position i and a key at position j <= i: a bias by distance
+//   chunk > 0      position i sees j only if i / chunk == j / chunk (chunks counted from position 0 of the sequence),
+//                  beside j <= i and beside a window, if there is one
+//
+// All of it in float, on both libraries.
+#pragma once
+#include <hip/hip_runtime.h>
+
+struct ScoreMod {
+  float cap;
+  const float* r1;
+  const float* r2;
+  int chunk;
+};
+
+// the first position that a token at position p may see
+__host__ __device__ __forceinline__ int reach_lo(int p, int window, int chunk) {
+  int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  if (chunk > 0 && p >= 0) {
+    const int c = p / chunk * chunk;
+    lo = c > lo ? c : lo;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ bool score_mod_on(const ScoreMod& m) { return m.cap > 0.f || m.r1 != nullptr; }
+
+// s: the scaled score; dist = i - j (taken as 0 where the key lies ahead of the query: such a key is masked anyway)
+__device__ __forceinline__ float mod_score(float s, float cap, bool biased, float r1, float r2, int dist) {
+  if (cap > 0.f) s = cap * tanhf(s / cap);
+  if (biased) s -= r1 * log1pf(r2 * (float)(dist > 0 ? dist : 0));
+  return s;
+}

@@ -37,6 +37,11 @@ int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const in
         hipStream_t st);
 int tq_moe_combine(const float* y, const int* pair_slot, const float* weights, int topk, const float* shared,
         int S, int64_t shared_stride, const float* gate, float* out, int T, int H, hipStream_t st);
+int tq_embed_pos(const int* tokens, const int* positions, const void* table, const void* pos_table, int wtype, float* x,
+        int T, int H, float scale, hipStream_t st);
+int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y, const int* pair_slot,
+        const float* weights, int topk, const float* gate, const void* wd, float eps_d, const void* w, int wtype,
+        float eps, const int* rows, int R, void* out, float* out32, int H, hipStream_t st);
 // gemm_generic.hip: the plain multiply-add product (both libraries)
 int tq_gemm_generic(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
         int wtype, int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
@@ -64,18 +69,43 @@ int tq_gemm_f32(const void* a, int64_t lda, const int* a_rows, int a_gather, con
 int tq_attention_generic(const void* q, const void* k_pool, const void* v_pool, const int* positions,
         const int* seq_of_token, const int* block_table, int bt_stride, int page_size, int64_t page_stride, int T,
         int nh, int nkv, int hd, int window, float scale, void* out, hipStream_t st);
+int tq_attention_generic_mod(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+        const int* seq_of_token, const int* block_table, int bt_stride, int page_size, int64_t page_stride, int T,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        void* out, hipStream_t st);
+// (the *_mod forms of the attention entry points take what score_mod.h describes: a cap on scores, a bias by
+// distance per head, chunks of positions)
 // attention_mfma.hip: bfloat16 attention on the matrix cores (bfloat16 library)
 int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end);
 int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, void* out, float* partial, int decode, int max_new,
         int max_end, hipStream_t st);
+int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+        const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st);
 // attention_f32.hip: float32 attention on the matrix cores (float32 library)
 int64_t tq_attention_f32_scratch(int B, int nh, int hd, int max_end);
 int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, void* out, void* partial, int decode, int max_new,
         int max_end, hipStream_t st);
+int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+        const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        void* out, void* partial, int decode, int max_new, int max_end, hipStream_t st);
+// delta_rule.hip: the gated delta rule over per-sequence state (both libraries)
+int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps);
+int tq_delta_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
+        const float* conv_w, int H, int G, int D, int V, int taps, int ra, int rg, float* qn, float* kn, float* vc,
+        float* beta, void* low, int T, hipStream_t st);
+int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, const float* ag,
+        const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
+        int64_t state_stride, int H, int G, int D, int V, int taps, int B, float* o_raw, hipStream_t st);
+int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w, float eps, const float* P,
+        const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V,
+        int taps, int ra, int rg, int T, int B, void* out, hipStream_t st);
 // moe.hip: router, choice of experts, order of pairs (both libraries)
 int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
         int* ids, float* weights, float* shared_gate, float* logits, int T, int H, hipStream_t st);
@@ -84,6 +114,11 @@ int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, int cap
 int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
         int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap, int* sorted_token,
         int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st);
+int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+        int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int T, int H, hipStream_t st);
+int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+        int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap,
+        int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st);
 // sampling.hip: greedy choice, negative log-likelihood, repetition penalty, temperature and top-p (both libraries; the two *_static entry points are declared in no_alloc.h)
 int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st);
 int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st);

@@ -32,10 +32,12 @@ def build_block(spec: LayerSpec) -> Part:
         cls = _REGISTRIES["block"][spec.block]
     except KeyError:
         raise ValueError(f"unknown block {spec.block!r}; known: {', '.join(sorted(_REGISTRIES['block']))}") from None
-    missing = [n for n in cls.slots if n not in spec.parts]
+    optional = getattr(cls, "optional", ())
+    missing = [n for n in cls.slots if n not in spec.parts and n not in optional]
     if missing:
         raise ValueError(f"block {spec.block!r} needs parts {missing}")
-    return cls(**{name: build_part(category, spec.parts[name]) for name, category in cls.slots.items()})
+    return cls(**{name: build_part(category, spec.parts[name]) for name, category in cls.slots.items()
+                  if name in spec.parts})
 
 
 def _bind(part: Part, spec: PartSpec, path: str, out: list[Binding]) -> None:
@@ -63,12 +65,17 @@ class CausalLM:
         self.bindings: list[Binding] = []
         for i, (ls, block) in enumerate(zip(plan.layers, self.blocks)):
             for name in block.slots:
-                _bind(getattr(block, name), ls.parts[name], f"layers.{i}.{name}", self.bindings)
+                if name in ls.parts:
+                    _bind(getattr(block, name), ls.parts[name], f"layers.{i}.{name}", self.bindings)
         _bind(self.final_norm, plan.final_norm, "final_norm", self.bindings)
         V, H = plan.vocab_size, plan.hidden_size
         self.bindings.append(Binding(self, "embedding", ParamSpec((V, H), role="table"), plan.embedding, "embedding"))
         if plan.lm_head is not None:
             self.bindings.append(Binding(self, "lm_head", ParamSpec((V, H)), plan.lm_head, "lm_head"))
+        self.position_table = None     # [max positions, H]: a learned vector per position, added to the embedded token
+        if plan.position_table is not None:
+            self.bindings.append(Binding(self, "position_table", ParamSpec((plan.max_positions, H), role="table"),
+                                         plan.position_table, "position_table"))
 
     # ------------------------------------------------------------ weights
     def tensor_table(self) -> dict:
@@ -119,12 +126,13 @@ class CausalLM:
             # same step part by part, for models with parts that the executor does not know, for whoever looks at
             # the layers (layer_hook) and for the profile, which puts an event behind every launch
             return ctx.native.forward(ctx)
-        x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale)
+        x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale,
+                      pos_table=self.position_table, positions=b.positions if self.position_table is not None else None)
         pending = None
         for entry, e in enumerate(self.schedule):
             pending = self.blocks[e.layer].forward(x, pending, ctx, entry)
             if ctx.layer_hook is not None:      # the stream with what the entry has left for the next norm to add
-                held = pending.materialize(self.act) if isinstance(pending, ops.GatheredSum) else pending
+                held = pending.materialize(self.act) if isinstance(pending, (ops.GatheredSum, ops.NormedDelta)) else pending
                 ctx.layer_hook(entry, x.clone() if held is None else x + held.sum(0), b)
         if b.n_want == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=x.device)
@@ -144,8 +152,10 @@ def model_from_config(config_json: dict, act: str) -> CausalLM:
 def load_model(model_dir: str, act: str = "bfloat16", device="cuda:0", f32_matrices: str = "bfloat16") -> CausalLM:
     """Reads config.json, picks the architecture from it, and loads model.safetensors by tensor name."""
     arch, cfg = config_from_dir(model_dir)
-    model = CausalLM(arch.plan(cfg), act, config=cfg)
     with SafetensorsFolder(model_dir) as folder:
+        if arch.complete is not None:       # sizes that only the tensors' shapes give
+            cfg = arch.complete(cfg, {n: tuple(e.shape) for n, e in folder.entries.items()})
+        model = CausalLM(arch.plan(cfg), act, config=cfg)
         model.load(folder, device, f32_matrices)
     return model
 

@@ -24,6 +24,8 @@ class NativeModel:
     def __init__(self, model, cache):
         self.model, self.cache = model, cache
         self.lib = host_api.library(model.act)
+        if getattr(model, "position_table", None) is not None:
+            raise ValueError("the step executor embeds tokens without a learned vector per position")
         layers = [b.native() for b in model.blocks]
         if any(l is None for l in layers):
             raise ValueError("a layer of the model has no form in the step executor")

@@ -7,6 +7,15 @@ softmax, weighted sum of values (:1908-1976); output projection (:2239-2240).  Q
 kv head h / (heads / kv_heads) (:1675-1679).  With a window a token reaches the last ``window``
 positions, itself included (:1646-1654).  With ``qk_norm_eps`` set, every head of q and of k is RMS-normed with
 weights of its own between the product and the rotation (:1111-1124), which this architecture does not use.
+
+Options for other designs, all off by default: ``position`` of kind "none" (no rotation: positions enter elsewhere);
+``score_cap`` c (a scaled score s becomes c tanh(s / c)); ``distance_bias`` (two numbers per head, r1 and r2:
+r1 ln(1 + r2 (i - j)) is taken off the score of query position i and key position j); ``chunk`` n (position i sees
+j <= i only if i // n == j // n, chunks counted from position 0 of the sequence); ``value_dim`` (values of another width
+than keys); ``separate_qkv`` (q, k, v and their biases are parameters of their own, joined when the part is prepared).
+With ``separate_qkv`` the heads are laid out at a kernel width that is the larger of key and value width rounded up to
+16: the added rows and columns of the matrices are zeros, which change no score and no output, and every head size
+then runs on the matrix-core kernels of both libraries.
 """
 from __future__ import annotations
 
@@ -24,12 +33,27 @@ class GroupedQueryAttention(Part):
     graph_safe = True
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, position,
                  qkv_bias: bool = False, out_bias: bool = False, window: int | None = None,
-                 scale: float | None = None, qk_norm_eps: float | None = None):
+                 scale: float | None = None, qk_norm_eps: float | None = None, score_cap: float | None = None,
+                 distance_bias: bool = False, chunk: int | None = None, value_dim: int | None = None,
+                 separate_qkv: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         if window is not None and window < 1:
             raise ValueError(f"window must be positive, got {window}")
+        if chunk is not None and chunk < 1:
+            raise ValueError(f"chunk must be positive, got {chunk}")
+        if score_cap is not None and not score_cap > 0:
+            raise ValueError(f"score_cap must be positive, got {score_cap}")
+        if value_dim not in (None, head_dim) and not separate_qkv:
+            raise ValueError("values of another width than keys need separate_qkv")
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.score_cap, self.has_distance_bias, self.chunk, self.separate_qkv = score_cap, distance_bias, chunk, separate_qkv
+        # what the checkpoint's heads measure (key width, value width); head_dim becomes the kernels' width
+        self.key_dim, self.value_dim = head_dim, head_dim if value_dim is None else value_dim
+        if separate_qkv:
+            self.head_dim = -(-max(self.key_dim, self.value_dim) // 16) * 16
+        self.r1 = self.r2 = None
+        self.q_weight = self.k_weight = self.v_weight = self.q_bias = self.k_bias = self.v_bias = None
         self.has_qkv_bias, self.has_out_bias, self.window = qkv_bias, out_bias, window
         self.qk_norm_eps = qk_norm_eps
         self.q_norm = self.k_norm = None
@@ -46,6 +70,18 @@ class GroupedQueryAttention(Part):
         return self.num_kv_heads * self.head_dim
 
     def param_specs(self):
+        if self.separate_qkv:
+            H, G, K, V, W = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.hidden_size
+            specs = {"q_weight": ParamSpec((H * K, W)), "k_weight": ParamSpec((G * K, W)), "v_weight": ParamSpec((G * V, W)),
+                     "out_weight": ParamSpec((W, H * V))}
+            if self.has_qkv_bias:
+                specs.update({"q_bias": ParamSpec((H * K,), role="bias"), "k_bias": ParamSpec((G * K,), role="bias"),
+                              "v_bias": ParamSpec((G * V,), role="bias")})
+            if self.has_out_bias:
+                specs["out_bias"] = ParamSpec((W,), role="bias")
+            if self.has_distance_bias:
+                specs.update({"r1": ParamSpec((H,), role="scale"), "r2": ParamSpec((H,), role="scale")})
+            return specs
         rows = self.q_size + 2 * self.kv_size
         splits = (self.q_size, self.kv_size, self.kv_size)
         specs = {
@@ -59,13 +95,40 @@ class GroupedQueryAttention(Part):
         if self.qk_norm_eps is not None:
             specs["q_norm"] = ParamSpec((self.head_dim,), role="scale")
             specs["k_norm"] = ParamSpec((self.head_dim,), role="scale")
+        if self.has_distance_bias:
+            specs.update({"r1": ParamSpec((self.num_heads,), role="scale"), "r2": ParamSpec((self.num_heads,), role="scale")})
         return specs
+
+    def prepare(self, device, act):
+        if self.has_distance_bias:      # they enter float arithmetic only
+            self.r1, self.r2 = self.r1.float().contiguous(), self.r2.float().contiguous()
+        if not self.separate_qkv or self.qkv_weight is not None:
+            return
+        D = self.head_dim
+
+        def heads_padded(t, heads, width):
+            """[heads * width, ...] -> [heads * D, ...], zeros behind each head's rows."""
+            out = t.new_zeros((heads, D, *t.shape[1:]))
+            out[:, :width] = t.view(heads, width, *t.shape[1:])
+            return out.view(heads * D, *t.shape[1:])
+
+        H, G, K, V = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        self.qkv_weight = torch.cat([heads_padded(self.q_weight, H, K), heads_padded(self.k_weight, G, K),
+                                     heads_padded(self.v_weight, G, V)])
+        if self.has_qkv_bias:
+            self.qkv_bias = torch.cat([heads_padded(self.q_bias, H, K), heads_padded(self.k_bias, G, K),
+                                       heads_padded(self.v_bias, G, V)])
+        if V != D:
+            out = self.out_weight.new_zeros((self.hidden_size, H, D))
+            out[:, :, :V] = self.out_weight.view(self.hidden_size, H, V)
+            self.out_weight = out.view(self.hidden_size, H * D).contiguous()
+        self.q_weight = self.k_weight = self.v_weight = self.q_bias = self.k_bias = self.v_bias = None
 
     def children(self):
         return {"position": self.position}
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window, chunk=self.chunk)
 
     def state_need(self):
         return None
@@ -74,6 +137,8 @@ class GroupedQueryAttention(Part):
         from ..csrc import host_api
         if self.qk_norm_eps is not None:        # the executor has no form with a norm of the heads
             return None
+        if self.score_cap is not None or self.has_distance_bias or self.chunk is not None or self.separate_qkv:
+            return None                         # nor one with changed scores or chunks
         table = self.position.table(self.qkv_weight.device)
         if table.dtype != torch.float32 or not table.is_contiguous() or table.numel() * 2 != self.position.rotary_dim:
             return None
@@ -96,5 +161,6 @@ class GroupedQueryAttention(Part):
             q = ops.rope_kv_write(qkv, *rope, runs=b.runs())
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
-                          self.window, self.scale, ctx.act, runs=b.runs())
+                          self.window, self.scale, ctx.act, runs=b.runs(), softcap=self.score_cap,
+                          distance_bias=(self.r1, self.r2) if self.has_distance_bias else None, chunk=self.chunk)
         return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)

@@ -47,11 +47,13 @@ class ParamSpec:
 class CacheNeed:
     """Keys and values per position: ``window`` None keeps all positions, else the last ``window``.
     ``head_dim`` is the width of a key row; ``value_dim`` that of a value row (None: the same; 0: no values are
-    kept, one row per position and kv head only)."""
+    kept, one row per position and kv head only).  ``chunk`` n: a token sees only the positions of its own chunk of n
+    (counted from position 0), so what lies before the chunk of the next token need not be kept."""
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
+    chunk: int | None = None
 
     @property
     def value_width(self) -> int:

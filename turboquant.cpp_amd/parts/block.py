@@ -48,3 +48,42 @@ class PreNormBlock(Part):
         want32 = getattr(self.ffn, "wants_f32", False)
         normed, normed32 = self.ffn_norm.forward(x, pending, ctx, want_f32=want32)
         return self.ffn.forward(normed, normed32, ctx)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Part):
+    """A norm before and a norm after every part: ``x += norm_b(mixer(norm_a(x))); x += norm_d(ffn(norm_c(x)))``, the
+    feed-forward half optional (``ffn``, ``ffn_norm`` and ``ffn_post_norm`` None: the layer is its mixer alone).  A
+    part's output travels to the next norm wrapped with the weights of the norm it has to pass first
+    (``ops.NormedDelta``), and that norm's kernel norms it, adds it into the stream and norms the stream in one pass."""
+    graph_safe = True
+    slots = {"mixer_norm": "norm", "mixer": "mixer", "mixer_post_norm": "norm", "ffn_norm": "norm", "ffn": "ffn",
+             "ffn_post_norm": "norm"}
+    optional = ("ffn_norm", "ffn", "ffn_post_norm")
+
+    def __init__(self, mixer_norm, mixer, mixer_post_norm, ffn_norm=None, ffn=None, ffn_post_norm=None):
+        if len({ffn_norm is None, ffn is None, ffn_post_norm is None}) != 1:
+            raise ValueError("a layer has a feed-forward with both its norms, or none of the three")
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ffn_norm, self.ffn, self.ffn_post_norm = ffn_norm, ffn, ffn_post_norm
+
+    def children(self):
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "mixer_post_norm": self.mixer_post_norm,
+                 "ffn_norm": self.ffn_norm, "ffn": self.ffn, "ffn_post_norm": self.ffn_post_norm}
+        return {k: v for k, v in parts.items() if v is not None}
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def forward(self, x, pending, ctx, entry):
+        from ..csrc import ops
+        normed, _ = self.mixer_norm.forward(x, pending, ctx)
+        pending = ops.NormedDelta(self.mixer.forward(normed, ctx, entry), self.mixer_post_norm.weight, self.mixer_post_norm.eps)
+        if self.ffn is None:
+            return pending
+        want32 = getattr(self.ffn, "wants_f32", False)
+        normed, normed32 = self.ffn_norm.forward(x, pending, ctx, want_f32=want32)
+        return ops.NormedDelta(self.ffn.forward(normed, normed32, ctx), self.ffn_post_norm.weight, self.ffn_post_norm.eps)

@@ -7,7 +7,8 @@ Sparse (/root/reference/src/engine/tq_moe.c:600-1059): router logits in float32,
 winning ties, weights from a softmax; every chosen expert is the dense formula with its own matrices, summed
 with its weight in the order chosen; the shared expert, scaled by ``sigmoid(x . shared_scale)``, is added
 last.  ``renormalize`` false keeps the softmax over all experts un-normalised for the chosen ones; true is
-the reference's softmax over the chosen logits.
+the reference's softmax over the chosen logits.  ``groups`` (count, keep): the experts form ``count`` equal groups of
+neighbours, a group's score is the largest score in it, and only experts of the ``keep`` best groups can be chosen.
 """
 from __future__ import annotations
 
@@ -61,9 +62,16 @@ class SparseMoE(Part):
     wants_f32 = True    # the router reads the normalised activations in float32
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,
-                 shared_gated: bool = True, renormalize: bool = False, activation: str = "silu"):
+                 shared_gated: bool = True, renormalize: bool = False, activation: str = "silu",
+                 groups: tuple[int, int] | None = None):
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must be within 1..num_experts {num_experts}")
+        if groups is not None:
+            count, keep = groups
+            if count < 1 or num_experts % count or not 1 <= keep <= count or top_k > keep * (num_experts // count):
+                raise ValueError(f"{count} groups of which {keep} are kept do not fit {num_experts} experts with {top_k} per token")
+            groups = None if count == 1 else (int(count), int(keep))
+        self.groups = groups
         if activation not in ops.GATES:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(sorted(ops.GATES))}")
         self.activation = activation
@@ -92,6 +100,8 @@ class SparseMoE(Part):
     def native(self):
         from ..csrc import host_api
         w = host_api.weight
+        if self.groups is not None:      # the executor chooses among all experts
+            return None
         return host_api.MoeFfnDesc(self.hidden_size, self.num_experts, self.top_k, self.expert_size, self.shared_size,
                                    int(self.renormalize), ops.GATES[self.activation], w(self.router),
                                    w(self.shared_scale if self.shared_gated else None), w(self.expert_gate), w(self.expert_up),
@@ -101,7 +111,7 @@ class SparseMoE(Part):
         T = normed.shape[0]
         unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate)
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
-                                  self.top_k, self.renormalize, unit, ctx.act)
+                                  self.top_k, self.renormalize, unit, ctx.act, groups=self.groups)
         if self.shared_size > 0 and T <= 16 and unit == 16:
             # a handful of tokens: the shared expert's two products ride in the launches of the routed experts'
             _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()

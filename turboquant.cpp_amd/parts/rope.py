@@ -48,3 +48,23 @@ class RotaryEncoding(Part):
 
     def prepare(self, device, act):
         self.table(device)
+
+
+@register_part("position", "none")
+class NoRotation(Part):
+    """No rotation of queries and keys: for models whose positions enter elsewhere (a learned vector added to the
+    embedding, a bias on the scores).  A mixer sees an empty table and a rotary width of 0."""
+    graph_safe = True
+    pairing_code = 0
+    rotary_dim = 0
+
+    def __init__(self):
+        self._table = None
+
+    def table(self, device) -> torch.Tensor:
+        if self._table is None or self._table.device != torch.device(device):
+            self._table = torch.zeros((1,), dtype=torch.float32, device=device)[:0]
+        return self._table
+
+    def prepare(self, device, act):
+        self.table(device)
