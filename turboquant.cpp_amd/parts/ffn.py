@@ -111,7 +111,8 @@ class SparseMoE(Part):
         T = normed.shape[0]
         unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate)
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
-                                  self.top_k, self.renormalize, unit, ctx.act, groups=self.groups)
+                                  self.top_k, self.renormalize, unit, ctx.act,
+                                  **({} if self.groups is None else {"groups": self.groups}))
         if self.shared_size > 0 and T <= 16 and unit == 16:
             # a handful of tokens: the shared expert's two products ride in the launches of the routed experts'
             _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
