@@ -9,6 +9,12 @@ chosen tokens to the host, exactly what the generation loop runs.  Prints one JS
     python bench.py --dtype float32 --workload unequal      # true 32-bit: 64 prompts of 1 to 2,048 tokens, 64 steps
 
 time the other two workloads: a batch of prompts of unequal lengths in one prompt step, then decode steps.
+
+    python bench.py --design felepel [--design-sizes small,medium] [--layers 8]
+
+times the Felepel design (delta-rule and chunked-attention layers, experts chosen within groups) beside Qwen2-MoE at
+equal sizes: prompt steps of 512 and 2,048 tokens, decode steps at batch 1 and 8, and where each model's time goes,
+kernel by kernel.  The default run and its line are not touched by it.
 """
 from __future__ import annotations
 
@@ -232,6 +238,119 @@ def unequal_workload(sizes: str, act: str, layers: int | None, wl: dict) -> dict
 
 
 
+# ---------------------------------------------------------------- the Felepel design beside Qwen2-MoE at equal sizes
+# name -> width, heads, kv heads of the attention, head size, experts, groups, kept groups, experts per token, expert width
+DESIGN_SIZES = {
+    "small": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=32, groups=4, keep=2, top=4, ff=768, vocab=32000),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=64, groups=8, keep=4, top=4, ff=1408, vocab=32000),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=32, groups=4, keep=2, top=2, ff=4096, vocab=32000),
+}
+
+
+def felepel_config(z: dict, layers: int, max_positions: int) -> dict:
+    """`layers` layers in the order delta rule, attention, attention, each with tensors of its own, so that the model has
+    as many matrices of the same sizes as the Qwen2-MoE model beside it."""
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": z["groups"], "keep": z["keep"]}}}
+    delta = {"type": "channel_delta", "mlp": moe,
+             "mixer": {"heads": z["heads"], "kv_heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4,
+                       "decay_rank": 64, "gate_rank": 64}}
+    attn = {"type": "attention", "mlp": moe,
+            "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                      "scale": z["dim"] ** -0.5, "softcap": 50.0, "mask": {"size": 1024}}}
+    out = []
+    for i in range(layers):
+        out.append(dict(delta if i % 3 == 0 else attn))
+    return {"architecture": "Felepel", "vocab": z["vocab"], "width": z["width"], "max_positions": max_positions,
+            "norm": {"eps": 1e-5}, "layers": out}
+
+
+def qwen_config_like(z: dict, layers: int, max_positions: int) -> dict:
+    return dict(A27B, vocab_size=z["vocab"], hidden_size=z["width"], num_hidden_layers=layers, num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], moe_intermediate_size=z["ff"],
+                shared_expert_intermediate_size=0, num_experts=z["experts"], num_experts_per_tok=z["top"],
+                max_window_layers=layers, max_position_embeddings=max_positions)
+
+
+def design_comparison(args) -> int:
+    import torch
+    from turboquant_cpp_amd.csrc import ops
+    from turboquant_cpp_amd.engine.model import random_model
+    from turboquant_cpp_amd.engine.step import Engine
+    act, dev = args.dtype, "cuda:0"
+    short = "bf16" if act == "bfloat16" else "fp32"
+    layers = args.layers or 6
+    context, prompts_at, batches = 2048, (512, 2048), (1, 8)
+    out = {"metric": "Felepel beside Qwen2-MoE at equal sizes: prompt and decode tok/s, and milliseconds by kernel",
+           "unit": "tok/s", "dtype": short, "layer_runs": layers, "data": "synthetic", "sizes": {}}
+
+    def measure(cfg):
+        model = random_model(cfg, seed=2, act=act, device=dev)
+        V = model.plan.vocab_size
+        gen = torch.Generator().manual_seed(5)
+        rec = {"weights_gb": round(model.weight_bytes / 1e9, 2), "prefill": {}, "decode": {}, "kernels_ms": {}}
+        for T in prompts_at:
+            engine = Engine(model, max_tokens=T + 64, page_size=64, max_slots=1)
+            prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+            best = None
+            for _ in range(4):
+                slot = engine.open(1)
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                engine.step(slot, [prompt])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t
+                engine.close(slot)
+                best = dt if best is None else min(best, dt)
+            rec["prefill"][str(T)] = {"tok_s": round(T / best, 1), "ms": round(best * 1e3, 3)}
+            # where the time goes: part by part on one stream, an event behind every launch
+            executor, engine.native, engine.side_stream = engine.native, None, None
+            slot = engine.open(1)
+            ops.profile_begin()
+            engine.step(slot, [prompt])
+            prof = ops.profile_end()
+            engine.close(slot)
+            engine.native = executor
+            rec["kernels_ms"][f"prefill_{T}"] = {k: [n, round(ms, 3)] for k, (n, ms) in sorted(prof["kernels"].items())}
+            del engine
+        for B in batches:
+            steps, warm = 32, 4
+            engine = Engine(model, max_tokens=(context + 64) * B, page_size=64, max_slots=B)
+            slots = engine.open(B)
+            for sl in slots:
+                engine.step([sl], [torch.randint(0, V, (context - steps - warm,), generator=gen).tolist()])
+            tokens = torch.randint(0, V, (B,), generator=gen, dtype=torch.int32).to(dev)
+            for _ in range(warm):
+                tokens = ops.argmax(engine.step_from_device(slots, tokens), act)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(steps):
+                tokens = ops.argmax(engine.step_from_device(slots, tokens), act)
+            torch.cuda.synchronize()
+            sec = (time.perf_counter() - t) / steps
+            rec["decode"][f"b{B}_ctx{context}"] = {"tok_s": round(B / sec, 1), "ms_per_step": round(sec * 1e3, 4)}
+            graphs, engine.graphs, executor, engine.native = engine.graphs, None, engine.native, None
+            ops.profile_begin()
+            engine.step_from_device(slots, tokens)
+            prof = ops.profile_end()
+            engine.graphs, engine.native = graphs, executor
+            rec["kernels_ms"][f"decode_b{B}"] = {k: [n, round(ms, 3)] for k, (n, ms) in sorted(prof["kernels"].items())}
+            engine.close(slots)
+            del engine
+        del model
+        torch.cuda.empty_cache()
+        return rec
+
+    for name in args.design_sizes.split(","):
+        z = DESIGN_SIZES[name]
+        out["sizes"][name] = {"config": z,
+                              "felepel": measure(felepel_config(z, layers, context + 64)),
+                              "qwen2_moe": measure(qwen_config_like(z, layers, context + 64))}
+        print(f"[bench] {name} done", file=sys.stderr, flush=True)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -265,12 +384,19 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--no-workloads", action="store_true",
                     help="leave out the two workloads of unequal prompts that the default run adds under \"workloads\"")
+    ap.add_argument("--design", default=None, choices=["felepel"],
+                    help="time this design beside Qwen2-MoE at equal sizes instead of the default workload")
+    ap.add_argument("--design-sizes", default="small,medium", help="of " + ", ".join(DESIGN_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
         return 2
     if args.probe:
         return probe()
+    if args.design:
+        from turboquant_cpp_amd.csrc import ops as _ops
+        _ops.library(args.dtype)
+        return design_comparison(args)
 
     import torch
     from turboquant_cpp_amd.csrc import ops

@@ -157,7 +157,7 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][D
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
-          s[g][jt][v] = mod_score(s[g][jt][v] * cm.scale, cm.cap, cm.biased, cm.r1[g], cm.r2[g], p_q[g] - key);
+          s[g][jt][v] = mod_score_fast(s[g][jt][v] * cm.scale, cm.cap, cm.biased, cm.r1[g], cm.r2[g], p_q[g] - key);
         }
     scale2 = LOG2E;
   }

@@ -38,8 +38,8 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // ------------------------------------------------------------------------------------------ per token
-// grid (T), block 256: a wave takes the "units" of its token in turn: the G query heads, the G key heads, the H
-// value heads, and one unit for beta and the low-rank activations.  An input before the token's run comes from the
+// grid (T, units / 4), block 256: a wave takes one "unit" of its token: one of the G query heads, the G key heads, the H
+// value heads, or the unit of beta and the low-rank activations.  An input before the token's run comes from the
 // state: the token is the c-th of its run if c of the taps - 1 tokens before it in the packed arrays have its slot
 // (c < taps - 1), and then input i - d (d > c) is the state's (d - c)-th most recent.
 __global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict__ P, const int* __restrict__ slot_of_token,
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict
   const float* hist = state + (size_t)slot * state_stride + (size_t)H * D * V;      // [C][K - 1]
   const float* row = P + (size_t)t * NP;
   const int units = 2 * G + H + 1;
-  for (int u = wave; u < units; u += 4) {
+  for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
     if (u == units - 1) {
       for (int h = lane; h < H; h += TQ_WAVE) beta[(size_t)t * H + h] = sigmoid_f(row[C + h]);
       for (int i = lane; i < dm.ra + dm.rg; i += TQ_WAVE)
@@ -91,24 +91,54 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict
   }
 }
 
+// ------------------------------------------------------------------------------------------ decays of a long step
+// ag[t][h D + i] <- exp(-exp(a_log[h]) * softplus(ag[t][h D + i] + dt_bias[h D + i])), in place, for the first H D
+// columns of every row: what the recurrence multiplies the state's rows by.  A step of many tokens works them out here,
+// once and in parallel; the recurrence of a short step does it as it stages its tokens.
+__global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ ag, const float* __restrict__ a_log,
+                                                          const float* __restrict__ dt_bias, int HD, int D, int AGW,
+                                                          int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % HD);
+  float* at = ag + (i / HD) * AGW + c;
+  *at = expf(-expf(a_log[c / D]) * softplus_f(*at + dt_bias[c]));
+}
+
 // ------------------------------------------------------------------------------------------ the recurrence
-// grid (H * col_blocks, B), block NSEG * cols: lane (col, seg) keeps rows 16 seg .. 16 seg + 15 of value channel col.
-// ag [T][H D + H V]: the decay's and the gate's second products; a_log [H], dt_bias [H D] float.
+// Sums over the NSEG lanes that share a value channel (neighbours, aligned): within quads, then the two quads of
+// eight lanes, then the two eights of a row of sixteen.  Every lane ends up with the total; the order is fixed.
+template <int NSEG>
+__device__ __forceinline__ float seg_sum(float v) {
+#define TQ_DPP_ADD(ctrl) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xf, 0xf, false))
+  if (NSEG >= 2) TQ_DPP_ADD(0xB1);        // quad_perm [1, 0, 3, 2]
+  if (NSEG >= 4) TQ_DPP_ADD(0x4E);        // quad_perm [2, 3, 0, 1]
+  if (NSEG >= 8) TQ_DPP_ADD(0x141);       // row_half_mirror
+  if (NSEG >= 16) TQ_DPP_ADD(0x140);      // row_mirror
+#undef TQ_DPP_ADD
+  return v;
+}
+
+// grid (H * col_blocks, B), block NSEG * cols rounded up to whole waves: lane (col, seg) keeps rows 16 seg .. 16 seg + 15
+// of value channel col.  The run's tokens pass through two LDS buffers in chunks of C = min(16, 8 block / DP) tokens:
+// while a chunk is worked through, the next one's values are on their way from memory into registers (8 of q, k and
+// decay per thread, 16 / NSEG of v), and go into the other buffer afterwards; one barrier a chunk.
+// ag [T][H D + H V]: the decay's and the gate's second products; decayed: the first H D columns already hold the decays
+// (delta_decay_kernel), else they hold what a_log [H] and dt_bias [H D] still have to be applied to.
+#define DR_STAGE 8
 template <int NSEG>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                          const float* __restrict__ vc, const float* __restrict__ beta,
                                                          const float* __restrict__ ag, const float* __restrict__ a_log,
-                                                         const float* __restrict__ dt_bias,
+                                                         const float* __restrict__ dt_bias, int decayed,
                                                          const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
                                                          float* __restrict__ state, int64_t state_stride, DeltaDims dm,
                                                          int cols, int col_blocks, float* __restrict__ o_raw) {
   constexpr int DP = DR_ROWS * NSEG;
+  constexpr int EV = 16 / NSEG;             // values of v per thread and chunk, at the most
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  float* qs = lds;                          // [DR_CHUNK][DP]
-  float* ks = qs + DR_CHUNK * DP;
-  float* gs = ks + DR_CHUNK * DP;
-  float* vs = gs + DR_CHUNK * DP;           // [DR_CHUNK][cols]
-  float* bs = vs + DR_CHUNK * cols;         // [DR_CHUNK]
+  const int C = min(DR_CHUNK, DR_STAGE * (int)blockDim.x / DP);
+  const int buf_floats = 3 * C * DP + C * cols + DR_CHUNK;
   const int H = dm.H, G = dm.G, D = dm.D, V = dm.V;
   const int h = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks, b = blockIdx.y;
   const int gq = h / (H / G);
@@ -125,28 +155,70 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
   }
   const float rate = expf(a_log[h]);
   const int AGW = H * D + H * V;
-  for (int c0 = 0; c0 < n; c0 += DR_CHUNK) {
-    const int nc = min(DR_CHUNK, n - c0);
-    __syncthreads();
-    for (int idx = tid; idx < nc * DP; idx += blockDim.x) {
-      const int c = idx / DP, r = idx % DP;
-      const size_t t = (size_t)(t0 + c0 + c);
-      float q = 0.f, k = 0.f, g = 1.f;
-      if (r < D) {
-        q = qn[t * G * D + (size_t)gq * D + r];
-        k = kn[t * G * D + (size_t)gq * D + r];
-        g = expf(-rate * softplus_f(ag[t * AGW + (size_t)h * D + r] + dt_bias[h * D + r]));
+
+  float rq[DR_STAGE], rk[DR_STAGE], rg[DR_STAGE], rv[EV], rb = 0.f;
+  // asks memory for the chunk that starts at token c0 of the run
+  auto fetch = [&](int c0) {
+    const int nc = min(C, n - c0);
+#pragma unroll
+    for (int j = 0; j < DR_STAGE; ++j) {
+      const int idx = tid + j * (int)blockDim.x, c = idx / DP, r = idx % DP;
+      rq[j] = rk[j] = 0.f;
+      rg[j] = decayed ? 1.f : INFINITY;      // a row beyond D keeps its zeros: decay 1 (softplus(-inf) = 0 gives the same)
+      if (c < nc && r < D) {
+        const size_t t = (size_t)(t0 + c0 + c);
+        rq[j] = qn[t * G * D + (size_t)gq * D + r];
+        rk[j] = kn[t * G * D + (size_t)gq * D + r];
+        rg[j] = ag[t * AGW + (size_t)h * D + r] + (decayed ? 0.f : dt_bias[h * D + r]);
       }
-      qs[idx] = q;
-      ks[idx] = k;
-      gs[idx] = g;
     }
-    for (int idx = tid; idx < nc * cols; idx += blockDim.x) {
-      const int c = idx / cols, j = cb * cols + idx % cols;
-      vs[idx] = j < V ? vc[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + j] : 0.f;
+#pragma unroll
+    for (int j = 0; j < EV; ++j) {
+      const int idx = tid + j * (int)blockDim.x, c = idx / cols, jj = cb * cols + idx % cols;
+      rv[j] = c < nc && jj < V ? vc[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + jj] : 0.f;
     }
-    if (tid < nc) bs[tid] = beta[(size_t)(t0 + c0 + tid) * H + h];
-    __syncthreads();
+    if (tid < nc) rb = beta[(size_t)(t0 + c0 + tid) * H + h];
+  };
+  // puts what fetch brought into buffer `at`
+  auto stage = [&](float* at, int c0) {
+    const int nc = min(C, n - c0);
+    float* qs = at;
+    float* ks = qs + C * DP;
+    float* gs = ks + C * DP;
+    float* vs = gs + C * DP;
+    float* bs = vs + C * cols;
+#pragma unroll
+    for (int j = 0; j < DR_STAGE; ++j) {
+      const int idx = tid + j * (int)blockDim.x;
+      if (idx < nc * DP) {
+        qs[idx] = rq[j];
+        ks[idx] = rk[j];
+        gs[idx] = decayed ? rg[j] : (rg[j] == INFINITY ? 1.f : expf(-rate * softplus_f(rg[j])));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < EV; ++j) {
+      const int idx = tid + j * (int)blockDim.x;
+      if (idx < nc * cols) vs[idx] = rv[j];
+    }
+    if (tid < nc) bs[tid] = rb;
+  };
+
+  if (n > 0) {
+    fetch(0);
+    stage(lds, 0);
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int c0 = 0; c0 < n; c0 += C, cur ^= 1) {
+    const int nc = min(C, n - c0);
+    const bool more = c0 + C < n;
+    if (more) fetch(c0 + C);
+    const float* qs = lds + cur * buf_floats;
+    const float* ks = qs + C * DP;
+    const float* gs = ks + C * DP;
+    const float* vs = gs + C * DP;
+    const float* bs = vs + C * cols;
     for (int c = 0; c < nc; ++c) {
       const float* qr = qs + c * DP + seg * DR_ROWS;
       const float* kr = ks + c * DP + seg * DR_ROWS;
@@ -162,18 +234,17 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
         d2 = fmaf(s[i], q, d2);
         d3 = fmaf(kk[i], q, d3);
       }
-#pragma unroll
-      for (int o = NSEG / 2; o > 0; o >>= 1) {
-        d1 += __shfl_xor(d1, o, TQ_WAVE);
-        d2 += __shfl_xor(d2, o, TQ_WAVE);
-        d3 += __shfl_xor(d3, o, TQ_WAVE);
-      }
+      d1 = seg_sum<NSEG>(d1);
+      d2 = seg_sum<NSEG>(d2);
+      d3 = seg_sum<NSEG>(d3);
       const float u = bs[c] * (vs[c * cols + (cl < cols ? cl : 0)] - d1);
 #pragma unroll
       for (int i = 0; i < DR_ROWS; ++i) s[i] = fmaf(kk[i], u, s[i]);
       // the read-out of the state that holds this token's write: (g S)^T q + u (k . q)
       if (col_ok && seg == 0) o_raw[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + col] = fmaf(u, d3, d2);
     }
+    if (more) stage(lds + (cur ^ 1) * buf_floats, c0 + C);
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
@@ -185,8 +256,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
 }
 
 // ------------------------------------------------------------------------------------------ norm, gate, new inputs
-// grid (T + B), block 256.  Blocks 0 .. T - 1: a wave per head of its token: o / rms(o) * w * sigmoid(gate).
-// Blocks T ..: the convolution's state of one sequence: its last taps - 1 inputs, those of this run and, where the run
+// grid (T + B, Y), block 256.  Blocks 0 .. T - 1 of x: a wave per head of its token: o / rms(o) * w * sigmoid(gate).
+// Blocks T ..: the convolution's state of one sequence, its channels dealt over y: its last taps - 1 inputs, those of this run and, where the run
 // is shorter, the most recent of the old state before them.
 __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const float* __restrict__ ag,
                                                         const float* __restrict__ norm_w, float eps,
@@ -198,7 +269,7 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
   if ((int)blockIdx.x < T) {
     const int t = blockIdx.x, wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
     const int AGW = H * D + H * V;
-    for (int h = wave; h < H; h += 4) {
+    for (int h = blockIdx.y * 4 + wave; h < H; h += 4 * gridDim.y) {
       const float* o = o_raw + (size_t)t * H * V + (size_t)h * V;
       float ss = 0.f;
       for (int j = lane; j < V; j += TQ_WAVE) ss += o[j] * o[j];
@@ -214,7 +285,7 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
   const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0;
   const int C = dd_channels(dm), NP = dd_np(dm);
   float* hist = state + (size_t)slots[b] * state_stride + (size_t)H * D * V;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
     float* hc = hist + (size_t)c * (K - 1);
     // new[m], m = 0 .. K - 2 oldest first, is the input K - 1 - m tokens before the run's end
     for (int m = 0; m < K - 1; ++m) {
@@ -246,19 +317,21 @@ TQ_API int tq_delta_prep(const float* P, const int* slot_of_token, const float* 
   if (T <= 0) return 0;
   const DeltaDims d{H, G, D, V, taps, ra, rg};
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
-  hipLaunchKernelGGL(delta_prep_kernel, dim3(T), dim3(256), 0, st, P, slot_of_token, state, state_stride, conv_w, d, qn,
+  const int units = 2 * G + H + 1;
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(T, (units + 3) / 4 < 65535 ? (units + 3) / 4 : 65535), dim3(256), 0, st, P, slot_of_token, state, state_stride, conv_w, d, qn,
                      kn, vc, beta, (act_t*)low);
   TQ_LAUNCH_CHECK();
   return 0;
 }
 
-// The recurrence over runs of tokens, one run per sequence (cu_seqlens [B + 1], slots [B]); the state rows are read
-// and written.  o_raw [T][H V] float.
-TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, const float* ag,
+// The recurrence over runs of tokens, one run per sequence (cu_seqlens [B + 1], slots [B], T tokens in all); the state
+// rows are read and written.  o_raw [T][H V] float.  In a step of many tokens the first H D columns of ag are replaced
+// by the decays they stand for (nothing else reads them afterwards).
+TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, float* ag,
                          const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
-                         int64_t state_stride, int H, int G, int D, int V, int taps, int B, float* o_raw,
+                         int64_t state_stride, int H, int G, int D, int V, int taps, int T, int B, float* o_raw,
                          hipStream_t st) {
-  if (B <= 0) return 0;
+  if (B <= 0 || T <= 0) return 0;
   const DeltaDims d{H, G, D, V, taps, 1, 1};
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
   if (B > 65535) return TQ_ERR_UNSUPPORTED;
@@ -268,12 +341,21 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
   const int col_blocks = (V + cols - 1) / cols;
   // whole waves, so that the lanes of a value channel always lie in one
   const int threads = (nseg * cols + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
-  const size_t shmem = ((size_t)3 * DR_CHUNK * DR_ROWS * nseg + (size_t)DR_CHUNK * cols + DR_CHUNK) * sizeof(float);
+  const int dp = DR_ROWS * nseg;
+  const int chunk = DR_CHUNK < DR_STAGE * threads / dp ? DR_CHUNK : DR_STAGE * threads / dp;
+  const size_t shmem = (size_t)2 * (3 * chunk * dp + chunk * cols + DR_CHUNK) * sizeof(float);
+  // the decays of a long step are worked out beforehand, once for all blocks of value channels
+  const int decayed = T > 16 * B || T >= 256;
+  if (decayed) {
+    const int64_t total = (int64_t)T * H * D;
+    hipLaunchKernelGGL(delta_decay_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ag, a_log, dt_bias,
+                       H * D, D, H * D + H * V, total);
+  }
 #define TQ_SCAN(NS)                                                                                                   \
   if (shmem > 48 * 1024)                                                                                              \
     (void)hipFuncSetAttribute((const void*)delta_scan_kernel<NS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
   hipLaunchKernelGGL(delta_scan_kernel<NS>, dim3(H * col_blocks, B), dim3(threads), shmem, st, qn, kn, vc, beta, ag,   \
-                     a_log, dt_bias, cu_seqlens, slots, state, state_stride, d, cols, col_blocks, o_raw)
+                     a_log, dt_bias, decayed, cu_seqlens, slots, state, state_stride, d, cols, col_blocks, o_raw)
   switch (nseg) {
     case 1: TQ_SCAN(1); break;
     case 2: TQ_SCAN(2); break;
@@ -294,7 +376,7 @@ TQ_API int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w
   if (T <= 0 || B <= 0) return 0;
   const DeltaDims d{H, G, D, V, taps, ra, rg};
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
-  hipLaunchKernelGGL(delta_out_kernel, dim3(T + B), dim3(256), 0, st, o_raw, ag, norm_w, eps, P, cu_seqlens, slots, state,
+  hipLaunchKernelGGL(delta_out_kernel, dim3(T + B, (H + 3) / 4 < 65535 ? (H + 3) / 4 : 65535), dim3(256), 0, st, o_raw, ag, norm_w, eps, P, cu_seqlens, slots, state,
                      state_stride, d, T, (act_t*)out);
   TQ_LAUNCH_CHECK();
   return 0;

@@ -70,7 +70,7 @@ _SIGNATURES = {
     "tq_delta_prep": [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
                       _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_delta_scan": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int,
-                      _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_delta_out": [_c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -451,6 +451,16 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
     return q
 
 
+_ZERO_ANGLES: dict = {}
+
+
+def _zero_angles(device, n: int) -> torch.Tensor:
+    key = (str(device), n)
+    if key not in _ZERO_ANGLES:
+        _ZERO_ANGLES[key] = torch.zeros((n,), dtype=torch.float32, device=device)
+    return _ZERO_ANGLES[key]
+
+
 def qkv_rope_write(a: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: torch.Tensor | None, positions: torch.Tensor,
                    seq_of_token: torch.Tensor, block_table: torch.Tensor, inv_freq: torch.Tensor, pairing: int,
                    rotary_dim: int, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, layer_offset: int,
@@ -462,6 +472,11 @@ def qkv_rope_write(a: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: torch.Te
     k = "qkv_rope_write"
     lib = library(act)
     T, K = a.shape
+    if (rotary_dim == 0 and T <= 16 and head_dim % 32 == 0 and hasattr(lib, "tq_qkv_rope_write")
+            and _use_mfma(act, a, qkv_weight, K)):
+        # no rotation at all: angles of zero turn nothing (cosine 1, sine 0: a * 1 - b * 0 is a to the bit), so the
+        # one launch whose workgroups rotate and store what they have summed serves such a mixer as well
+        inv_freq, pairing, rotary_dim = _zero_angles(a.device, head_dim // 2), 0, head_dim
     fused = (hasattr(lib, "tq_qkv_rope_write") and T <= 16 and pairing == 0 and rotary_dim == head_dim
              and head_dim % 32 == 0 and _use_mfma(act, a, qkv_weight, K)
              and (qkv_bias is None or qkv_bias.dtype in _WTYPE))
@@ -1051,7 +1066,8 @@ def delta_scan(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch
                a_log: torch.Tensor, dt_bias: torch.Tensor, runs: dict, state: torch.Tensor, dims: DeltaDims, act):
     """The recurrence over each sequence's run of tokens, in order, from and into its row of ``state``:
     S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with g = exp(-exp(a_log) softplus(a + dt_bias))
-    from the first H*dim columns of ``ag`` [T, H*dim + H*vdim].  Returns o, float32 [T, H*vdim]."""
+    from the first H*dim columns of ``ag`` [T, H*dim + H*vdim] (which a step of many tokens overwrites with those g).
+    Returns o, float32 [T, H*vdim]."""
     k = "delta_scan"
     T = qn.shape[0]
     G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
@@ -1065,7 +1081,7 @@ def delta_scan(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch
     _check(runs["slots"], k, "slots", torch.int32, (B,))
     o = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)
     _run(k, library(act).tq_delta_scan(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(ag), _ptr(a_log), _ptr(dt_bias),
-                                       _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), B,
+                                       _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), T, B,
                                        _ptr(o), _stream()))
     return o
 

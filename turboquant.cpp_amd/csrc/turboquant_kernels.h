@@ -100,9 +100,9 @@ int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps);
 int tq_delta_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
         const float* conv_w, int H, int G, int D, int V, int taps, int ra, int rg, float* qn, float* kn, float* vc,
         float* beta, void* low, int T, hipStream_t st);
-int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, const float* ag,
+int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, float* ag,
         const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
-        int64_t state_stride, int H, int G, int D, int V, int taps, int B, float* o_raw, hipStream_t st);
+        int64_t state_stride, int H, int G, int D, int V, int taps, int T, int B, float* o_raw, hipStream_t st);
 int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w, float eps, const float* P,
         const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V,
         int taps, int ra, int rg, int T, int B, void* out, hipStream_t st);

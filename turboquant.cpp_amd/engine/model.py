@@ -126,8 +126,8 @@ class CausalLM:
             # same step part by part, for models with parts that the executor does not know, for whoever looks at
             # the layers (layer_hook) and for the profile, which puts an event behind every launch
             return ctx.native.forward(ctx)
-        x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale,
-                      pos_table=self.position_table, positions=b.positions if self.position_table is not None else None)
+        learned = {} if self.position_table is None else {"pos_table": self.position_table, "positions": b.positions}
+        x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale, **learned)
         pending = None
         for entry, e in enumerate(self.schedule):
             pending = self.blocks[e.layer].forward(x, pending, ctx, entry)

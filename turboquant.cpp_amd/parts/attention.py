@@ -147,6 +147,17 @@ class GroupedQueryAttention(Part):
                                       host_api.weight(self.qkv_weight), host_api.weight(self.qkv_bias),
                                       host_api.weight(self.out_weight), host_api.weight(self.out_bias), table.data_ptr())
 
+    def _score_options(self) -> dict:
+        """What the attention kernels are told beyond the plain formula; nothing for a mixer that leaves it all off."""
+        opts = {}
+        if self.score_cap is not None:
+            opts["softcap"] = self.score_cap
+        if self.has_distance_bias:
+            opts["distance_bias"] = (self.r1, self.r2)
+        if self.chunk is not None:
+            opts["chunk"] = self.chunk
+        return opts
+
     def forward(self, normed, ctx, entry):
         b, kv = ctx.batch, ctx.kv(entry)
         rope = (b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device), self.position.pairing_code,
@@ -161,6 +172,5 @@ class GroupedQueryAttention(Part):
             q = ops.rope_kv_write(qkv, *rope, runs=b.runs())
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
-                          self.window, self.scale, ctx.act, runs=b.runs(), softcap=self.score_cap,
-                          distance_bias=(self.r1, self.r2) if self.has_distance_bias else None, chunk=self.chunk)
+                          self.window, self.scale, ctx.act, runs=b.runs(), **self._score_options())
         return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)
