@@ -119,87 +119,103 @@ __device__ __forceinline__ float seg_sum(float v) {
   return v;
 }
 
-// grid (H * col_blocks, B), block NSEG * cols rounded up to whole waves: lane (col, seg) keeps rows 16 seg .. 16 seg + 15
-// of value channel col.  The run's tokens pass through two LDS buffers in chunks of C = min(16, 8 block / DP) tokens:
+// grid (H * col_blocks, B), block NSEG * LC rounded up to whole waves: lane (lc, seg) keeps rows 16 seg .. 16 seg + 15 of the
+// CPT value channels lc, lc + LC, ... of its block of cols = CPT * LC: several channels to a lane give it chains of
+// multiply-adds that do not wait for each other, and one read of q, k and the decays from LDS serves them all.  The run's tokens pass through two LDS buffers in chunks of C = min(16, 8 block / DP) tokens:
 // while a chunk is worked through, the next one's values are on their way from memory into registers (8 of q, k and
 // decay per thread, 16 / NSEG of v), and go into the other buffer afterwards; one barrier a chunk.
-// ag [T][H D + H V]: the decay's and the gate's second products; decayed: the first H D columns already hold the decays
-// (delta_decay_kernel), else they hold what a_log [H] and dt_bias [H D] still have to be applied to.
+// ag [T][H D + H V]: the decay's and the gate's second products; DECAYED: the first H D columns already hold the decays
+// (delta_decay_kernel), else they hold what a_log [H] and dt_bias [H D] still have to be applied to (a kernel of its own
+// for each, so that the one for long steps carries no exponentials).
 #define DR_STAGE 8
-template <int NSEG>
+// A lane's 16 rows of q, k and decays lie 20 floats from its neighbour's in LDS, not 16: the lanes of a wave that read
+// different rows then hit different banks (blocks 80 bytes apart start at banks 0, 20, 8, 28, 16, 4, 24, 12).
+#define DR_PAD 20
+template <int NSEG, int CPT, bool DECAYED>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                          const float* __restrict__ vc, const float* __restrict__ beta,
                                                          const float* __restrict__ ag, const float* __restrict__ a_log,
-                                                         const float* __restrict__ dt_bias, int decayed,
+                                                         const float* __restrict__ dt_bias,
                                                          const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
                                                          float* __restrict__ state, int64_t state_stride, DeltaDims dm,
                                                          int cols, int col_blocks, float* __restrict__ o_raw) {
-  constexpr int DP = DR_ROWS * NSEG;
-  constexpr int EV = 16 / NSEG;             // values of v per thread and chunk, at the most
+  constexpr int DP = DR_ROWS * NSEG, RL = DR_PAD * NSEG;      // rows of a token, and the floats they take in LDS
+  constexpr int EV = 16 * CPT / NSEG > 0 ? 16 * CPT / NSEG : 1;      // values of v per thread and chunk, at the most
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int C = min(DR_CHUNK, DR_STAGE * (int)blockDim.x / DP);
-  const int buf_floats = 3 * C * DP + C * cols + DR_CHUNK;
+  // (a multiple of four floats, so that either buffer's rows of q, k and decays can be read 16 bytes at a time)
+  const int buf_floats = 3 * C * RL + (C * cols + 3) / 4 * 4 + DR_CHUNK;
   const int H = dm.H, G = dm.G, D = dm.D, V = dm.V;
   const int h = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks, b = blockIdx.y;
   const int gq = h / (H / G);
-  const int tid = threadIdx.x, seg = tid % NSEG, cl = tid / NSEG;
-  const int col = cb * cols + cl;
-  const bool col_ok = cl < cols && col < V;
+  const int tid = threadIdx.x, seg = tid % NSEG, lc = tid / NSEG;
+  const int LC = cols / CPT;                 // lanes' columns in the block; cols is a multiple of CPT
+  int cloc[CPT];                             // this lane's channels within the block (0 where it has none)
+  bool col_ok[CPT];
   const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0;
   float* S = state + (size_t)slots[b] * state_stride + (size_t)h * D * V;
-  float s[DR_ROWS];
+  float s[CPT][DR_ROWS];
 #pragma unroll
-  for (int i = 0; i < DR_ROWS; ++i) {
-    const int r = seg * DR_ROWS + i;
-    s[i] = col_ok && r < D ? S[(size_t)r * V + col] : 0.f;
+  for (int j = 0; j < CPT; ++j) {
+    const int cl = lc + j * LC;
+    col_ok[j] = lc < LC && cb * cols + cl < V;
+    cloc[j] = col_ok[j] ? cl : 0;
+#pragma unroll
+    for (int i = 0; i < DR_ROWS; ++i) {
+      const int r = seg * DR_ROWS + i;
+      s[j][i] = col_ok[j] && r < D ? S[(size_t)r * V + cb * cols + cl] : 0.f;
+    }
   }
   const float rate = expf(a_log[h]);
   const int AGW = H * D + H * V;
 
   float rq[DR_STAGE], rk[DR_STAGE], rg[DR_STAGE], rv[EV], rb = 0.f;
-  // asks memory for the chunk that starts at token c0 of the run
+  // Asks memory for the chunk that starts at token c0 of the run.  Every load is unconditional, from an address that
+  // is clamped into the chunk, and what lies outside is replaced when the values are staged: a load under a condition
+  // is followed by a wait for it (its value is merged with the other branch's right away), and the loads of a chunk
+  // then go out one by one, a memory latency each.
   auto fetch = [&](int c0) {
     const int nc = min(C, n - c0);
 #pragma unroll
     for (int j = 0; j < DR_STAGE; ++j) {
-      const int idx = tid + j * (int)blockDim.x, c = idx / DP, r = idx % DP;
-      rq[j] = rk[j] = 0.f;
-      rg[j] = decayed ? 1.f : INFINITY;      // a row beyond D keeps its zeros: decay 1 (softplus(-inf) = 0 gives the same)
-      if (c < nc && r < D) {
-        const size_t t = (size_t)(t0 + c0 + c);
-        rq[j] = qn[t * G * D + (size_t)gq * D + r];
-        rk[j] = kn[t * G * D + (size_t)gq * D + r];
-        rg[j] = ag[t * AGW + (size_t)h * D + r] + (decayed ? 0.f : dt_bias[h * D + r]);
-      }
+      const int idx = tid + j * (int)blockDim.x, c = min(idx / DP, nc - 1), r = min(idx % DP, D - 1);
+      const size_t t = (size_t)(t0 + c0 + c);
+      rq[j] = qn[t * G * D + (size_t)gq * D + r];
+      rk[j] = kn[t * G * D + (size_t)gq * D + r];
+      rg[j] = ag[t * AGW + (size_t)h * D + r];
     }
 #pragma unroll
     for (int j = 0; j < EV; ++j) {
-      const int idx = tid + j * (int)blockDim.x, c = idx / cols, jj = cb * cols + idx % cols;
-      rv[j] = c < nc && jj < V ? vc[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + jj] : 0.f;
+      const int idx = tid + j * (int)blockDim.x, c = min(idx / cols, nc - 1), jj = min(cb * cols + idx % cols, V - 1);
+      rv[j] = vc[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + jj];
     }
-    if (tid < nc) rb = beta[(size_t)(t0 + c0 + tid) * H + h];
+    rb = beta[(size_t)(t0 + c0 + min(tid, nc - 1)) * H + h];
   };
-  // puts what fetch brought into buffer `at`
+  // puts what fetch brought into buffer `at`; a row beyond D keeps its zeros (q = k = 0, decay 1)
   auto stage = [&](float* at, int c0) {
     const int nc = min(C, n - c0);
     float* qs = at;
-    float* ks = qs + C * DP;
-    float* gs = ks + C * DP;
-    float* vs = gs + C * DP;
-    float* bs = vs + C * cols;
+    float* ks = qs + C * RL;
+    float* gs = ks + C * RL;
+    float* vs = gs + C * RL;
+    float* bs = vs + (C * cols + 3) / 4 * 4;
 #pragma unroll
     for (int j = 0; j < DR_STAGE; ++j) {
-      const int idx = tid + j * (int)blockDim.x;
+      const int idx = tid + j * (int)blockDim.x, r = idx % DP;
       if (idx < nc * DP) {
-        qs[idx] = rq[j];
-        ks[idx] = rk[j];
-        gs[idx] = decayed ? rg[j] : (rg[j] == INFINITY ? 1.f : expf(-rate * softplus_f(rg[j])));
+        const bool row = r < D;
+        const int to = idx / DP * RL + r / DR_ROWS * DR_PAD + r % DR_ROWS;
+        qs[to] = row ? rq[j] : 0.f;
+        ks[to] = row ? rk[j] : 0.f;
+        float g = rg[j];
+        if constexpr (!DECAYED) g = expf(-rate * softplus_f(g + dt_bias[h * D + min(r, D - 1)]));
+        gs[to] = row ? g : 1.f;
       }
     }
 #pragma unroll
     for (int j = 0; j < EV; ++j) {
       const int idx = tid + j * (int)blockDim.x;
-      if (idx < nc * cols) vs[idx] = rv[j];
+      if (idx < nc * cols) vs[idx] = cb * cols + idx % cols < V ? rv[j] : 0.f;
     }
     if (tid < nc) bs[tid] = rb;
   };
@@ -214,43 +230,71 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
     const int nc = min(C, n - c0);
     const bool more = c0 + C < n;
     if (more) fetch(c0 + C);
-    const float* qs = lds + cur * buf_floats;
-    const float* ks = qs + C * DP;
-    const float* gs = ks + C * DP;
-    const float* vs = gs + C * DP;
-    const float* bs = vs + C * cols;
-    for (int c = 0; c < nc; ++c) {
-      const float* qr = qs + c * DP + seg * DR_ROWS;
-      const float* kr = ks + c * DP + seg * DR_ROWS;
-      const float* gr = gs + c * DP + seg * DR_ROWS;
-      float kk[DR_ROWS];
-      float d1 = 0.f, d2 = 0.f, d3 = 0.f;
+    const float* qs = (const float*)__builtin_assume_aligned(lds + cur * buf_floats, 16);
+    const float* ks = qs + C * RL;
+    const float* gs = ks + C * RL;
+    const float* vs = gs + C * RL;
+    const float* bs = vs + (C * cols + 3) / 4 * 4;
+    // One token: the rows' decays, the two sums over the state's rows, the write, the read-out.  The token's q, k and
+    // decays (qq, kk, gg) were read from LDS while the token before was worked through (two sets of registers taking
+    // turns, so that a read from LDS is never waited for right after it is asked).
+    auto load_token = [&](int c, float (&qq)[DR_ROWS], float (&kk)[DR_ROWS], float (&gg)[DR_ROWS]) {
+      const float* qr = (const float*)__builtin_assume_aligned(qs + c * RL + seg * DR_PAD, 16);
+      const float* kr = (const float*)__builtin_assume_aligned(ks + c * RL + seg * DR_PAD, 16);
+      const float* gr = (const float*)__builtin_assume_aligned(gs + c * RL + seg * DR_PAD, 16);
 #pragma unroll
       for (int i = 0; i < DR_ROWS; ++i) {
+        qq[i] = qr[i];
         kk[i] = kr[i];
-        const float q = qr[i];
-        s[i] *= gr[i];
-        d1 = fmaf(s[i], kk[i], d1);
-        d2 = fmaf(s[i], q, d2);
-        d3 = fmaf(kk[i], q, d3);
+        gg[i] = gr[i];
       }
-      d1 = seg_sum<NSEG>(d1);
-      d2 = seg_sum<NSEG>(d2);
-      d3 = seg_sum<NSEG>(d3);
-      const float u = bs[c] * (vs[c * cols + (cl < cols ? cl : 0)] - d1);
+    };
+    auto one_token = [&](int c, const float (&qq)[DR_ROWS], const float (&kk)[DR_ROWS], const float (&gg)[DR_ROWS]) {
+      float d1[CPT], d2[CPT], d3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < DR_ROWS; ++i) s[i] = fmaf(kk[i], u, s[i]);
-      // the read-out of the state that holds this token's write: (g S)^T q + u (k . q)
-      if (col_ok && seg == 0) o_raw[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + col] = fmaf(u, d3, d2);
+      for (int j = 0; j < CPT; ++j) d1[j] = d2[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < DR_ROWS; ++i) {
+        d3 = fmaf(kk[i], qq[i], d3);
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+          s[j][i] *= gg[i];
+          d1[j] = fmaf(s[j][i], kk[i], d1[j]);
+          d2[j] = fmaf(s[j][i], qq[i], d2[j]);
+        }
+      }
+      d3 = seg_sum<NSEG>(d3);
+      const float bt = bs[c];
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) {
+        const float u = bt * (vs[c * cols + cloc[j]] - seg_sum<NSEG>(d1[j]));
+#pragma unroll
+        for (int i = 0; i < DR_ROWS; ++i) s[j][i] = fmaf(kk[i], u, s[j][i]);
+        // the read-out of the state that holds this token's write: (g S)^T q + u (k . q)
+        const float o = fmaf(u, d3, seg_sum<NSEG>(d2[j]));
+        if (col_ok[j] && seg == 0) o_raw[(size_t)(t0 + c0 + c) * H * V + (size_t)h * V + cb * cols + cloc[j]] = o;
+      }
+    };
+    float qa[DR_ROWS], ka[DR_ROWS], ga[DR_ROWS], qb[DR_ROWS], kb[DR_ROWS], gb[DR_ROWS];
+    load_token(0, qa, ka, ga);
+    for (int c = 0; c < nc; c += 2) {
+      if (c + 1 < nc) load_token(c + 1, qb, kb, gb);
+      one_token(c, qa, ka, ga);
+      if (c + 1 < nc) {
+        if (c + 2 < nc) load_token(c + 2, qa, ka, ga);
+        one_token(c + 1, qb, kb, gb);
+      }
     }
     if (more) stage(lds + (cur ^ 1) * buf_floats, c0 + C);
     __syncthreads();
   }
-  if (col_ok) {
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    if (!col_ok[j]) continue;
 #pragma unroll
     for (int i = 0; i < DR_ROWS; ++i) {
       const int r = seg * DR_ROWS + i;
-      if (r < D) S[(size_t)r * V + col] = s[i];
+      if (r < D) S[(size_t)r * V + cb * cols + cloc[j]] = s[j][i];
     }
   }
 }
@@ -337,13 +381,22 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
   if (B > 65535) return TQ_ERR_UNSUPPORTED;
   int nseg = 1;
   while (nseg * DR_ROWS < D) nseg *= 2;
-  const int cols = V < 256 / nseg ? V : 256 / nseg;
+  // value channels per lane: as many of 4, 2, 1 as still leave the head's lanes a whole wave
+  // (measured on 16 heads of 128 x 128, one sequence of 2,048 tokens: 0.51 us a token with one channel per lane, 0.65 with
+  // two, 1.0 with four, since fewer lanes then share the head's work; several channels pay where the step's sequences
+  // and heads alone give every compute unit its workgroups)
+  const int lanes_one = nseg * V;                                  // lanes a head takes with one channel per lane
+  const int64_t groups_one = (int64_t)B * H * ((lanes_one + 255) / 256);
+  int cpt = groups_one >= 2048 ? 4 : groups_one >= 1024 ? 2 : 1;
+  while (cpt > 1 && nseg * ((V + cpt - 1) / cpt) < TQ_WAVE) cpt /= 2;
+  const int lane_cols = (V + cpt - 1) / cpt < 256 / nseg ? (V + cpt - 1) / cpt : 256 / nseg;     // LC
+  const int cols = lane_cols * cpt;
   const int col_blocks = (V + cols - 1) / cols;
   // whole waves, so that the lanes of a value channel always lie in one
-  const int threads = (nseg * cols + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
+  const int threads = (nseg * lane_cols + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
   const int dp = DR_ROWS * nseg;
   const int chunk = DR_CHUNK < DR_STAGE * threads / dp ? DR_CHUNK : DR_STAGE * threads / dp;
-  const size_t shmem = (size_t)2 * (3 * chunk * dp + chunk * cols + DR_CHUNK) * sizeof(float);
+  const size_t shmem = (size_t)2 * (3 * chunk * DR_PAD * nseg + (chunk * cols + 3) / 4 * 4 + DR_CHUNK) * sizeof(float);
   // the decays of a long step are worked out beforehand, once for all blocks of value channels
   const int decayed = T > 16 * B || T >= 256;
   if (decayed) {
@@ -351,11 +404,26 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
     hipLaunchKernelGGL(delta_decay_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ag, a_log, dt_bias,
                        H * D, D, H * D + H * V, total);
   }
-#define TQ_SCAN(NS)                                                                                                   \
-  if (shmem > 48 * 1024)                                                                                              \
-    (void)hipFuncSetAttribute((const void*)delta_scan_kernel<NS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
-  hipLaunchKernelGGL(delta_scan_kernel<NS>, dim3(H * col_blocks, B), dim3(threads), shmem, st, qn, kn, vc, beta, ag,   \
-                     a_log, dt_bias, decayed, cu_seqlens, slots, state, state_stride, d, cols, col_blocks, o_raw)
+#define TQ_SCAN_WITH(NS, CP, DEC)                                                                                     \
+  do {                                                                                                                \
+    if (shmem > 48 * 1024)                                                                                            \
+      (void)hipFuncSetAttribute((const void*)delta_scan_kernel<NS, CP, DEC>,                                          \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                              \
+    hipLaunchKernelGGL((delta_scan_kernel<NS, CP, DEC>), dim3(H * col_blocks, B), dim3(threads), shmem, st, qn, kn,   \
+                       vc, beta, ag, a_log, dt_bias, cu_seqlens, slots, state, state_stride, d, cols, col_blocks,     \
+                       o_raw);                                                                                        \
+  } while (0)
+#define TQ_SCAN_AS(NS, CP)                   \
+  do {                                       \
+    if (decayed) TQ_SCAN_WITH(NS, CP, true); \
+    else TQ_SCAN_WITH(NS, CP, false);        \
+  } while (0)
+#define TQ_SCAN(NS)                  \
+  do {                               \
+    if (cpt == 4) TQ_SCAN_AS(NS, 4); \
+    else if (cpt == 2) TQ_SCAN_AS(NS, 2); \
+    else TQ_SCAN_AS(NS, 1);          \
+  } while (0)
   switch (nseg) {
     case 1: TQ_SCAN(1); break;
     case 2: TQ_SCAN(2); break;
@@ -363,6 +431,8 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
     case 8: TQ_SCAN(8); break;
     default: TQ_SCAN(16); break;
   }
+#undef TQ_SCAN_AS
+#undef TQ_SCAN_WITH
 #undef TQ_SCAN
   TQ_LAUNCH_CHECK();
   return 0;
