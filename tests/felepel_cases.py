@@ -51,11 +51,12 @@ CASES = {
         (attention(3, 3, 24, 8, chunk=17, softcap=None, scale=0.31), moe(5, 5, 36)),
         ("of", 1),
     ]),
-    # a width that is no multiple of four, two taps, one expert of one, the attention first
+    # a width that is no multiple of four, two taps, five and one (no convolution at all), one expert of one, the attention first
     "ragged": config(50, 67, [
         (attention(5, 5, 10, 10, chunk=64), moe(1, 1, 10)),
         (delta(2, 1, 40, 24, conv=2), moe(9, 2, 18, 3, 2)),
         (delta(3, 3, 8, 70, conv=5), None),
+        (delta(2, 2, 16, 8, conv=1), None),
     ]),
     # as a served model's layers might be laid out, small: heads of 64, one kv head, groups, looped layers
     "regular": config(128, 256, [

@@ -60,6 +60,10 @@ def test_what_config_json_may_leave_out_and_may_not():
             at[path[-1]] = value
         with pytest.raises(ConfigError, match=message):
             config_from_dict(bad)
+    ahead = copy.deepcopy(base)
+    ahead["layers"].insert(0, {**ahead["layers"][1], "weights_of": 2})      # a layer may run the tensors of a later one
+    _, c3 = config_from_dict(ahead)
+    assert c3.layers[0].weights_of == 2 and c3.layers[0].type == "channel_delta"
     bad = copy.deepcopy(base)
     bad["layers"].append({**bad["layers"][0], "weights_of": 1})       # an attention layer with a delta layer's weights
     with pytest.raises(ConfigError, match="weights of layer 1"):

@@ -132,25 +132,30 @@ def config_from_json(data: dict) -> FelepelConfig:
         kind = entry.get("type")
         require(kind in (ATTENTION, DELTA), f"layers[{i}].type {kind!r} is not implemented ({ATTENTION} and {DELTA} are)")
         of = entry.get("weights_of")
-        require(of is None or (isinstance(of, int) and not isinstance(of, bool) and 0 <= of < i),
-                f"layers[{i}].weights_of must name an earlier layer, got {of!r}")
-        layer = FelepelLayer(kind, _mixer(kind, _object(entry, "mixer", where), where + ".mixer"),
-                             _mlp(_object(entry, "mlp", where, optional=True), where + ".mlp"), of)
-        if of is not None:
-            src = cfg.layers[of]
-            require(src.weights_of is None, f"layers[{i}].weights_of names layer {of}, which has no tensors of its own")
-            require(src.type == kind, f"layers[{i}] is {kind} but uses the weights of layer {of}, which is {src.type}")
-            if isinstance(layer.mixer, DeltaMixer):     # the ranks are the tensors' and so the other layer's
-                layer.mixer.decay_rank, layer.mixer.gate_rank = src.mixer.decay_rank, src.mixer.gate_rank
-            require(layer.mixer == src.mixer and layer.mlp == src.mlp,
-                    f"layers[{i}] uses the weights of layer {of} but its sizes or constants differ")
-        cfg.layers.append(layer)
+        require(of is None or (isinstance(of, int) and not isinstance(of, bool) and 0 <= of < len(layers) and of != i),
+                f"layers[{i}].weights_of must name another layer, got {of!r}")
+        cfg.layers.append(FelepelLayer(kind, _mixer(kind, _object(entry, "mixer", where), where + ".mixer"),
+                                       _mlp(_object(entry, "mlp", where, optional=True), where + ".mlp"), of))
+    for i, layer in enumerate(cfg.layers):      # a layer on another's tensors: the other has its own, and the two agree
+        of = layer.weights_of
+        if of is None:
+            continue
+        src = cfg.layers[of]
+        require(src.weights_of is None, f"layers[{i}].weights_of names layer {of}, which has no tensors of its own")
+        require(src.type == layer.type, f"layers[{i}] is {layer.type} but uses the weights of layer {of}, which is {src.type}")
+        if isinstance(layer.mixer, DeltaMixer):     # the ranks are the tensors' and so the other layer's
+            layer.mixer.decay_rank, layer.mixer.gate_rank = src.mixer.decay_rank, src.mixer.gate_rank
+        require(layer.mixer == src.mixer and layer.mlp == src.mlp,
+                f"layers[{i}] uses the weights of layer {of} but its sizes or constants differ")
     return cfg
 
 
 def complete(cfg: FelepelConfig, shapes: dict) -> FelepelConfig:
-    """The sizes that only the checkpoint's tensors give: the ranks of the delta rule's low-rank products."""
+    """The sizes that only the checkpoint's tensors give: the ranks of the delta rule's low-rank products, and how many
+    positions the table of learned position vectors has if that is not what config.json says."""
     cfg = copy.deepcopy(cfg)
+    if "pos" in shapes and len(shapes["pos"]) == 2:
+        cfg.max_positions = int(shapes["pos"][0])
     for i, layer in enumerate(cfg.layers):
         if not isinstance(layer.mixer, DeltaMixer):
             continue
