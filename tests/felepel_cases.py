@@ -67,7 +67,42 @@ CASES = {
 }
 
 
-def tensors(cfg: dict, seed: int, peaky: float = 1.0, memory: float = 0.0) -> dict[str, np.ndarray]:
+def random_case(seed: int) -> tuple[dict, tuple[int, int]]:
+    """A configuration drawn from sizes of many kinds (and the ranks of the delta rule's low-rank products, which only
+    the tensors' shapes carry)."""
+    rng = np.random.default_rng(7000 + seed)
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    divisors = lambda n: [d for d in range(1, n + 1) if n % d == 0]
+    width = pick([40, 56, 64, 90, 96, 120, 160, 200, 256, 320])
+
+    def mlp():
+        if rng.random() < 0.25:
+            return None
+        experts = pick([2, 4, 6, 8, 12, 16])
+        count = pick(divisors(experts))
+        keep = int(rng.integers(1, count + 1))
+        top = int(rng.integers(1, min(keep * (experts // count), 4) + 1))
+        return moe(experts, top, pick([8, 20, 24, 40, 64, 100]), count, keep)
+
+    layers = []
+    for i in range(int(rng.integers(2, 6))):
+        if i >= 1 and rng.random() < 0.3:
+            own = [j for j, l in enumerate(layers) if l[0] != "of"]
+            layers.append(("of", pick(own)))
+            continue
+        heads = pick([1, 2, 3, 4, 6, 8])
+        kv = pick(divisors(heads))
+        if rng.random() < 0.5:
+            dim = pick([4, 8, 12, 16, 24, 32, 40, 48, 64, 80, 96])
+            layers.append((attention(heads, kv, dim, pick([4, 8, 16, 24, 32, 48, 64, 72, 96]), scale=float(rng.uniform(0.5, 1.5)) * dim ** -0.5,
+                                     softcap=pick([None, 20.0, 50.0]), chunk=pick([None, 7, 32, 50, 64, 96, 130])), mlp()))
+        else:
+            layers.append((delta(heads, kv, pick([4, 8, 16, 20, 32, 48, 64]), pick([4, 8, 16, 24, 32, 64, 96]),
+                                 conv=pick([1, 2, 3, 4, 6])), mlp()))
+    return config(width, int(rng.integers(50, 500)), layers, max_positions=256), (pick([3, 8, 24]), pick([5, 16]))
+
+
+def tensors(cfg: dict, seed: int, peaky: float = 1.0, memory: float = 0.0, ranks: tuple[int, int] = (6, 10)) -> dict[str, np.ndarray]:
     """Random weights as float64 arrays whose values are bfloat16 numbers.  ``peaky`` scales the attention's query
     matrices, so that single keys decide a row of the softmax; ``memory`` is taken off A_log, so that the delta rule's
     state decays slowly and far tokens matter."""
@@ -100,7 +135,7 @@ def tensors(cfg: dict, seed: int, peaky: float = 1.0, memory: float = 0.0) -> di
             put(p + "mix.o", (W, H * V), (H * V) ** -0.5)
             put(p + "mix.o.b", (W,), 0.1)
         else:
-            ra, rg = 6, 10
+            ra, rg = ranks
             for n, rows in (("q", G * D), ("k", G * D), ("v", H * V)):
                 put(f"{p}mix.{n}", (rows, W), W ** -0.5)
                 put(f"{p}mix.{n}.conv", (rows, m["conv"]), 0.6)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import plain_felepel as plain
-from felepel_cases import CASES, tensors, tokens, write_folder
+from felepel_cases import CASES, random_case, tensors, tokens, write_folder
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -91,7 +91,7 @@ def test_whole_prompt(made, case):
         check(got, plain.forward(cfg, w, toks), what=f"{case}, {n} tokens")
 
 
-@pytest.mark.parametrize("case", ["regular", "odd"])
+@pytest.mark.parametrize("case", ["regular", "odd", "ragged"])
 def test_whole_prompt_bfloat16(made, case):
     d, cfg, w = made(case)
     eng = engine_of(d, "bfloat16")
@@ -99,6 +99,35 @@ def test_whole_prompt_bfloat16(made, case):
     slot = eng.open(1)
     got = eng.step(slot, [toks], [all_places(len(toks))])
     check(got, plain.forward(cfg, w, toks), "bfloat16", case)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_sizes_of_many_kinds(tmp_path, seed):
+    """Configurations drawn at random: a prompt in two portions and a few decoded tokens, two requests side by side, in
+    true 32-bit against the plain implementation at every position, and in bfloat16, where most positions are close."""
+    cfg, ranks = random_case(seed)
+    w = tensors(cfg, seed, ranks=ranks)
+    d = write_folder(str(tmp_path), cfg, w)
+    a, b = tokens(cfg, 140, seed), tokens(cfg, 31, 100 + seed)
+    wa, wb = plain.forward(cfg, w, a), plain.forward(cfg, w, b)
+    for dtype in ("float32", "bfloat16"):
+        eng = engine_of(d, dtype)
+        sa, sb = eng.open(2)
+        out = eng.step([sa, sb], [a[:70], b[:3]], [all_places(70), all_places(3)])
+        rows_a, rows_b = [out[:70]], [out[70:]]
+        out = eng.step([sa, sb], [a[70:130], b[3:]], [all_places(60), all_places(len(b) - 3)])
+        rows_a.append(out[:60])
+        rows_b.append(out[60:])
+        eng.close([sb])
+        rows_a += [eng.step([sa], [[t]]) for t in a[130:]]
+        ga, gb = torch.cat(rows_a), torch.cat(rows_b)
+        assert bool(torch.isfinite(ga).all()) and bool(torch.isfinite(gb).all())
+        if dtype == "float32":
+            check(ga, wa, what=f"seed {seed}: {json.dumps(cfg['layers'])}")
+            check(gb, wb, what=f"seed {seed}, second request")
+        else:
+            # (five layers of experts behind rounded activations: choices differ here and there, and stay differing)
+            assert np.median(errors(ga, wa)) < 0.1, f"seed {seed}: median {np.median(errors(ga, wa)):.3f}"
 
 
 def test_layers_one_by_one(made):
@@ -117,7 +146,7 @@ def test_layers_one_by_one(made):
 
 # ---------------------------------------------------------------- decoding, portions, batches
 @pytest.mark.parametrize("case,dtype", [("odd", "float32"), ("ragged", "float32"), ("regular", "float32"),
-                                        ("regular", "bfloat16")])
+                                        ("regular", "bfloat16"), ("odd", "bfloat16"), ("ragged", "bfloat16")])
 def test_prompt_then_token_by_token(made, case, dtype):
     """Most of a sequence in one step, the rest one token a step (the later steps replayed as graphs), across the
     edges of chunks and pages."""
@@ -376,6 +405,24 @@ def test_greedy_generation_through_the_entry_point(made):
         for j, tok in enumerate(g):
             row = rows[len(p) - 1 + j]
             assert row[tok] >= row.max() - 1e-3, f"token {j} of a prompt of {len(p)} is not the plain model's choice"
+
+
+def test_command_line(made):
+    """``bin/quant``: what it says of the folder, and greedy tokens that are the entry point's."""
+    from turboquant_cpp_amd import Model
+    d, cfg, w = made("regular", seed=5)
+    quant = os.path.join(ROOT, "bin", "quant")
+    info = subprocess.run([quant, d, "--info"], capture_output=True, text=True, timeout=300)
+    assert info.returncode == 0 and "Felepel" in info.stdout and "max_positions" in info.stdout, info.stderr[-1000:]
+    run = subprocess.run([quant, d, "-p", "5,17,3;8,1", "-n", "6", "-T", "0", "--rep-penalty", "1.0", "--dtype", "float32",
+                          "--json", "-M"], capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    with Model(d, dtype="float32", temperature=0.0, rep_penalty=1.0, max_tokens=6) as m:
+        want = m.generate([[5, 17, 3], [8, 1]])
+    got = [r["tokens"] for r in json.loads(run.stdout.strip().splitlines()[-1])]
+    assert got == want
+    c = subprocess.run([os.path.join(ROOT, "bin", "quant_c"), d, "-p", "5,17"], capture_output=True, text=True, timeout=300)
+    assert c.returncode == 2 and "bin/quant runs this model" in c.stderr
 
 
 def test_trace_runner_as_a_program(made, tmp_path):

@@ -365,7 +365,8 @@ int moe_ffn(Ctx& c, const tq_moe_ffn_desc& f, const void* normed, const float* n
   const bool gated = Is > 0 && f.shared_scale.ptr != nullptr;
   if (gated && f.shared_scale.wtype != f.router.wtype) return fail(TQ_ERR_BAD_ARG, "route: shared_scale must have the router's type");
   const int64_t n_pairs = (int64_t)T * k;
-  const int unit = expert_tile_rows(c, n_pairs, E, use_mfma(f.expert_gate, H));
+  // (the units that only the matrix-core product takes, where both of the experts' products run there)
+  const int unit = expert_tile_rows(c, n_pairs, E, use_mfma(f.expert_gate, H) && use_mfma(f.expert_down, I));
   int64_t cap = n_pairs + (E < n_pairs ? E : n_pairs) * (unit - 1);
   cap = (cap + unit - 1) / unit * unit;
   // outputs of the routing

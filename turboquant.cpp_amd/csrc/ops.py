@@ -550,7 +550,8 @@ TILE_PAIRS = 1024            # added to tile_rows 64: two units of one expert pe
 EXPERT_PAIRS_FROM = 48       # rows per expert on average from which units of 64 are taken two at a time
 
 
-def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
+def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor,
+                     w_behind: torch.Tensor | None = None) -> int:
     """Rows per tile (the padding unit of the row order) that suit a product over experts, by the pairs per expert on
     average.  Up to 5: 16, the streaming kernel, which passes an expert's matrices once per 16 of its rows.  Up to 10,
     where the bfloat16 matrix-core product runs: 32, the same kernel with two row tiles and two column tiles to a wave.
@@ -566,7 +567,9 @@ def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: to
     taken two at a time (expert_product_rows) are faster than either (60 experts of 1,408 x 2,048, both products:
     396 us against 448 at 205 rows per expert, 492 against 565 at 273, 841 against 949 at 546; 64 experts of
     2,560 x 3,584 at 1,650 rows each: a prompt step of 425 ms against 436 with units of 256)."""
-    mfma = _use_mfma(act, a, w, a.shape[1])
+    # (``w_behind``: the matrices of the product that follows on the same row order, over another k: the units that only
+    # the matrix-core product takes are chosen where both products run there)
+    mfma = _use_mfma(act, a, w, a.shape[1]) and (w_behind is None or _use_mfma(act, a, w_behind, w_behind.shape[-1]))
     if n_pairs <= (EXPERT_16_UPTO if mfma else 12) * num_experts:
         return 16
     if mfma and n_pairs <= EXPERT_32_UPTO * num_experts:

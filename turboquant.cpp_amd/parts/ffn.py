@@ -109,7 +109,8 @@ class SparseMoE(Part):
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
-        unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate)
+        unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate,
+                                    **({} if self.expert_size % 8 == 0 else {"w_behind": self.expert_down}))
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
                                   self.top_k, self.renormalize, unit, ctx.act,
                                   **({} if self.groups is None else {"groups": self.groups}))
