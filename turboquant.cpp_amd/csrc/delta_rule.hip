@@ -7,12 +7,13 @@
 // and silu.  Each head's o is then divided by its root mean square, multiplied by a weight per value channel and by a
 // sigmoid gate.  Everything here is float arithmetic on both libraries; the products around it are the library's.
 //
-// Three kernels, for prompts and for decoding alike (a decoded token is a run of one):
+// The kernels, for prompts and for decoding alike (a decoded token is a run of one):
 //   delta_prep   per token: convolution (its first inputs from the sequence's state), silu, unit vectors, beta, and
 //                the low-rank activations of the decay and the gate in the activation type, for the product behind
+//   delta_decay  (steps of many tokens) the decays of all tokens, in parallel, in place of what they are made from
 //   delta_scan   per (sequence, head, block of value channels): the recurrence over the run's tokens in order, the
-//                state in registers (16 key channels of one value channel per lane), tokens staged through LDS in
-//                chunks with their decays worked out in parallel
+//                state in registers (16 key channels of a value channel per lane), tokens staged through two LDS
+//                buffers in chunks; a short step works out its decays as it stages them
 //   delta_out    per token: norm and gate of every head; and per sequence: the convolution's new state
 //
 // A sequence's row of state (float): S as [H][D][V], then for every convolution channel (q's, k's, v's) its last

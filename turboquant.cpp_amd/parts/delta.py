@@ -14,8 +14,8 @@ per value channel (shared by the heads) and by sigmoid(W_g2 (W_g1 x)), and the h
 The sequence's state is one row of float32 per slot (``StateNeed``): S, then the convolution's last taps - 1 inputs of
 every channel.  Decays, gates, norms and the recurrence are float32 on both libraries; the products are the
 activation type's.  Six launches a step, prompt or decode: the product of all first projections, ``delta_prep``, the
-second product of decay and gate (one product over a block-diagonal matrix of both), ``delta_scan``, ``delta_out``,
-the output product.
+second product of decay and gate (one product over a block-diagonal matrix of both), ``delta_scan`` (which, in a step
+of many tokens, first works out all decays in a launch of their own), ``delta_out``, the output product.
 """
 from __future__ import annotations
 
