@@ -58,6 +58,14 @@ CASES = {
         (delta(3, 3, 8, 70, conv=5), None),
         (delta(2, 2, 16, 8, conv=1), None),
     ]),
+    # heads as wide as served models have them, and wider: key widths of 128, 192 and 256 (8 and 16 lanes to a value
+    # channel in the recurrence's kernel, the last with rows to spare), value widths beyond one block of lanes
+    "wide": config(256, 300, [
+        (delta(4, 2, 128, 128), moe(8, 2, 128, 4, 2)),
+        (attention(4, 1, 128, 128, chunk=64, softcap=50.0), None),
+        (delta(1, 1, 256, 40, conv=2), None),
+        (delta(2, 1, 192, 272, conv=3), None),
+    ]),
     # as a served model's layers might be laid out, small: heads of 64, one kv head, groups, looped layers
     "regular": config(128, 256, [
         (delta(4, 4, 32, 32), moe(8, 2, 64, 2, 1)),

@@ -91,7 +91,7 @@ def test_whole_prompt(made, case):
         check(got, plain.forward(cfg, w, toks), what=f"{case}, {n} tokens")
 
 
-@pytest.mark.parametrize("case", ["regular", "odd", "ragged"])
+@pytest.mark.parametrize("case", ["regular", "odd", "ragged", "wide"])
 def test_whole_prompt_bfloat16(made, case):
     d, cfg, w = made(case)
     eng = engine_of(d, "bfloat16")
@@ -146,7 +146,8 @@ def test_layers_one_by_one(made):
 
 # ---------------------------------------------------------------- decoding, portions, batches
 @pytest.mark.parametrize("case,dtype", [("odd", "float32"), ("ragged", "float32"), ("regular", "float32"),
-                                        ("regular", "bfloat16"), ("odd", "bfloat16"), ("ragged", "bfloat16")])
+                                        ("regular", "bfloat16"), ("odd", "bfloat16"), ("ragged", "bfloat16"),
+                                        ("wide", "float32"), ("wide", "bfloat16")])
 def test_prompt_then_token_by_token(made, case, dtype):
     """Most of a sequence in one step, the rest one token a step (the later steps replayed as graphs), across the
     edges of chunks and pages."""
