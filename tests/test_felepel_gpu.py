@@ -408,6 +408,35 @@ def test_greedy_generation_through_the_entry_point(made):
             assert row[tok] >= row.max() - 1e-3, f"token {j} of a prompt of {len(p)} is not the plain model's choice"
 
 
+def test_a_conversation_with_state_and_chunks(made, tmp_path):
+    """``Model.chat`` on a model with recurrent state and chunked groups: a turn that goes on runs only the new tokens; a
+    history that parts from the cached tokens starts over (a state has no earlier value); a saved conversation (pages,
+    rows of state, tokens) goes on in another model object with the same tokens."""
+    from turboquant_cpp_amd import Model
+    d, cfg, w = made("regular", seed=5)
+    opts = dict(dtype="float32", temperature=0.0, rep_penalty=1.0, max_tokens=5, context_length=512)
+    h1, extra, other, more = (tokens(cfg, n, 70 + n) for n in (70, 9, 150, 5))
+    with Model(d, **opts) as m, Model(d, **opts) as fresh:
+        brought = []
+        step = m.engine.step
+        m.engine.step = lambda slots, toks, *a, **k: (brought.append(len(toks[0])), step(slots, toks, *a, **k))[1]
+        out1 = m.chat(h1)
+        assert out1 == fresh.generate([h1])[0] and brought[0] == 70
+        del brought[:]
+        h2 = h1 + out1 + extra
+        out2 = m.chat(h2)
+        assert brought[0] == 1 + len(extra) and out2 == fresh.generate([h2])[0]
+        saved = str(tmp_path / "talk.kv")
+        m.save_context(saved)
+        del brought[:]
+        h3 = h1[:40] + other
+        assert m.chat(h3) == fresh.generate([h3])[0] and brought[0] == len(h3)
+        with Model(d, **opts) as later:
+            later.load_context(saved)
+            h4 = h2 + out2 + more
+            assert later.chat(h4) == fresh.generate([h4])[0]
+
+
 def test_command_line(made):
     """``bin/quant``: what it says of the folder, and greedy tokens that are the entry point's."""
     from turboquant_cpp_amd import Model
