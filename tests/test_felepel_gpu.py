@@ -130,6 +130,19 @@ def test_sizes_of_many_kinds(tmp_path, seed):
             assert np.median(errors(ga, wa)) < 0.1, f"seed {seed}: median {np.median(errors(ga, wa)):.3f}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_a_thousand_tokens(made, dtype):
+    """Long enough for the plain products of the bfloat16 path to go to the vendor's library, over many chunks and pages,
+    then decoded on."""
+    d, cfg, w = made("regular", seed=7)
+    eng = engine_of(d, dtype)
+    toks = tokens(cfg, 1010, 13)
+    want = plain.forward(cfg, w, toks)
+    slot = eng.open(1)
+    rows = [eng.step(slot, [toks[:1000]], [all_places(1000)])] + [eng.step(slot, [[t]]) for t in toks[1000:]]
+    check(torch.cat(rows), want, dtype, "1,000 tokens")
+
+
 def test_layers_one_by_one(made):
     """The residual stream behind every layer run, looped layers included."""
     d, cfg, w = made("odd")
