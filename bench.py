@@ -242,8 +242,8 @@ def unequal_workload(sizes: str, act: str, layers: int | None, wl: dict) -> dict
 # name -> width, heads, kv heads of the attention, head size, experts, groups, kept groups, experts per token, expert width
 DESIGN_SIZES = {
     "small": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=32, groups=4, keep=2, top=4, ff=768, vocab=32000),
-    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=64, groups=8, keep=4, top=4, ff=1408, vocab=32000),
-    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=32, groups=4, keep=2, top=2, ff=4096, vocab=32000),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=64, groups=8, keep=2, top=4, ff=1408, vocab=32000),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=32, groups=4, keep=1, top=2, ff=4096, vocab=32000),
 }
 
 

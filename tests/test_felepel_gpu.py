@@ -362,8 +362,9 @@ def test_experts_within_the_best_groups(E, top, count, keep):
 
 
 def test_delta_rule_kernels_with_a_state_carried_over(made):
-    """The mixer's three kernels against the plain function, the sequence cut in two runs so that the second starts
-    from the first one's state and convolution inputs, two sequences side by side in slots far apart."""
+    """The mixer's kernels against the plain function, the sequence cut in two runs so that the second starts from the
+    first one's state and convolution inputs, and one more token through the decode step's single kernel; two sequences
+    side by side in slots far apart."""
     from turboquant_cpp_amd.csrc import ops
     for case, layer in (("ragged", 1), ("ragged", 2), ("odd", 0)):
         _, cfg, w = made(case)
@@ -373,7 +374,7 @@ def test_delta_rule_kernels_with_a_state_carried_over(made):
         dims = ops.DeltaDims(H, G, D, V, K, ra, rg)
         rng = np.random.default_rng(layer)
         lens, slots = (23, 1), (5, 2)
-        hs = [rng.normal(size=(n + 9, cfg["width"])) for n in lens]
+        hs = [rng.normal(size=(n + 10, cfg["width"])) for n in lens]
         want = [plain.channel_delta(h, m, w, p, 1e-5, return_state=True) for h in hs]
         dev = "cuda"
         f32 = lambda a: torch.tensor(np.ascontiguousarray(a), dtype=torch.float32, device=dev)
@@ -383,18 +384,23 @@ def test_delta_rule_kernels_with_a_state_carried_over(made):
         w_low[:H * D, :ra], w_low[H * D:, ra:] = w[p + "a2"], w[p + "g2"]
         conv = f32(np.concatenate([w[p + n] for n in ("q.conv", "k.conv", "v.conv")]))
         outs = [[], []]
-        for run in range(2):
-            parts = [h[:n] if run == 0 else h[n:] for h, n in zip(hs, lens)]
+        for run in range(3):
+            parts = [h[:n] if run == 0 else h[n:n + 9] if run == 1 else h[n + 9:] for h, n in zip(hs, lens)]
             x = np.concatenate(parts)
             cu = np.cumsum([0] + [len(q) for q in parts])
             runs = {"cu_seqlens": torch.tensor(cu, dtype=torch.int32, device=dev),
-                    "slots": torch.tensor(slots, dtype=torch.int32, device=dev)}
+                    "slots": torch.tensor(slots, dtype=torch.int32, device=dev), "decode": run == 2}
             slot_of_token = torch.tensor(np.repeat(slots, [len(q) for q in parts]), dtype=torch.int32, device=dev)
             proj = f32(x @ w_in.T)
             qn, kn, vc, beta, low = ops.delta_prep(proj, slot_of_token, state, conv, dims, "float32")
-            ag = f32(low.double().cpu().numpy() @ w_low.T)
-            o = ops.delta_scan(qn, kn, vc, beta, ag, f32(w[p + "A_log"]), f32(w[p + "dt_bias"]), runs, state, dims, "float32")
-            out = ops.delta_out(o, ag, f32(w[p + "norm"]), 1e-5, proj, runs, state, dims, "float32")
+            if run == 2:
+                assert ops.delta_decode_fits(dims)
+                out = ops.delta_decode(qn, kn, vc, beta, low, f32(w_low), f32(w[p + "A_log"]), f32(w[p + "dt_bias"]),
+                                       f32(w[p + "norm"]), 1e-5, proj, runs, state, dims, "float32")
+            else:
+                ag = f32(low.double().cpu().numpy() @ w_low.T)
+                o = ops.delta_scan(qn, kn, vc, beta, ag, f32(w[p + "A_log"]), f32(w[p + "dt_bias"]), runs, state, dims, "float32")
+                out = ops.delta_out(o, ag, f32(w[p + "norm"]), 1e-5, proj, runs, state, dims, "float32")
             y = out.double().cpu().numpy() @ w[p + "o"].T
             for i in range(2):
                 outs[i].append(y[cu[i]:cu[i + 1]])

@@ -15,6 +15,8 @@
 //                state in registers (16 key channels of a value channel per lane), tokens staged through two LDS
 //                buffers in chunks; a short step works out its decays as it stages them
 //   delta_out    per token: norm and gate of every head; and per sequence: the convolution's new state
+//   delta_decode (steps of one token per sequence) the second low-rank products, decays, recurrence, norm, gate and the
+//                convolution's new state in one launch
 //
 // A sequence's row of state (float): S as [H][D][V], then for every convolution channel (q's, k's, v's) its last
 // taps - 1 inputs, oldest first.  Projections P [T][NP] (float): q (G D) | k (G D) | v (H V) | b (H) | a1 (ra) | g1 (rg).
@@ -341,6 +343,112 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
   }
 }
 
+// ------------------------------------------------------------------------------------------ one token per sequence
+// A decode step's form of what lies between delta_prep and the output product, in one launch: the second low-rank
+// products of this head's decay and gate (four lanes to a row of the block-diagonal matrix), the decays, the recurrence for the one token, the read-out's norm and gate, and the convolution's new state.
+// grid (H, B), block NSEG * V rounded up to whole waves (at most 1,024): lane (col, seg) keeps rows 16 seg .. 16 seg + 15
+// of value channel col, all of a head's value channels in one workgroup, so that their norm needs no second kernel.
+// The convolution's state of a head's own value channels is moved on by that head's workgroup, that of a q/k head by
+// the workgroup of the first head that reads it; delta_prep, which read the old state, has finished by then.
+template <int NSEG, class W>
+__global__ __launch_bounds__(1024) void delta_decode_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                                                            const float* __restrict__ vc, const float* __restrict__ beta,
+                                                            const act_t* __restrict__ low, const W* __restrict__ w_low,
+                                                            const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                                            const float* __restrict__ norm_w, float eps,
+                                                            const float* __restrict__ P, const int* __restrict__ cu_seqlens,
+                                                            const int* __restrict__ slots, float* __restrict__ state,
+                                                            int64_t state_stride, DeltaDims dm, act_t* __restrict__ out) {
+  constexpr int DP = DR_ROWS * NSEG, RL = DR_PAD * NSEG;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* qs = lds;                 // [RL] each: a lane's 16 rows 20 floats from its neighbour's
+  float* ks = qs + RL;
+  float* gs = ks + RL;
+  float* gate = gs + RL;           // [V]
+  float* lowv = gate + (dm.V + 3) / 4 * 4;      // [ra + rg]
+  float* red = lowv + (dm.ra + dm.rg + 3) / 4 * 4;      // one per wave
+  const int H = dm.H, G = dm.G, D = dm.D, V = dm.V, K = dm.taps, R = dm.ra + dm.rg;
+  const int h = blockIdx.x, b = blockIdx.y, gq = h / (H / G);
+  const int tid = threadIdx.x, seg = tid % NSEG, col = tid / NSEG;
+  const bool col_ok = col < V;
+  const size_t t = (size_t)cu_seqlens[b];
+  float* row = state + (size_t)slots[b] * state_stride;
+  for (int i = tid; i < R; i += blockDim.x) lowv[i] = to_f32(low[t * R + i]);
+  __syncthreads();
+  const float rate = expf(a_log[h]);
+  // The head's D rows of the decay's product and V rows of the gate's, four neighbouring lanes to a row: lane p of the
+  // four sums the elements p, p + 4, ... of the rank, and the four partial sums are added within the quad.
+  const int part = tid & 3, rows_a_pass = (int)blockDim.x >> 2;
+  for (int r0 = 0; r0 < D + V; r0 += rows_a_pass) {
+    const int r = r0 + (tid >> 2);
+    const bool live = r < D + V, decay = r < D;
+    float a = 0.f;
+    if (live) {
+      const W* wr = decay ? w_low + (size_t)(h * D + r) * R : w_low + (size_t)(H * D + h * V + (r - D)) * R + dm.ra;
+      const float* lv = decay ? lowv : lowv + dm.ra;
+      const int n = decay ? dm.ra : dm.rg;
+#pragma unroll 4
+      for (int j = part; j < n; j += 4) a = fmaf(to_f32(wr[j]), lv[j], a);
+    }
+    a = seg_sum<4>(a);
+    if (live && part == 0) {
+      if (decay) {
+        const int to = r / DR_ROWS * DR_PAD + r % DR_ROWS;
+        qs[to] = qn[t * G * D + (size_t)gq * D + r];
+        ks[to] = kn[t * G * D + (size_t)gq * D + r];
+        gs[to] = expf(-rate * softplus_f(a + dt_bias[h * D + r]));
+      } else {
+        gate[r - D] = a;
+      }
+    }
+  }
+  for (int r = D + tid; r < DP; r += blockDim.x) {      // rows beyond D keep their zeros
+    const int to = r / DR_ROWS * DR_PAD + r % DR_ROWS;
+    qs[to] = ks[to] = 0.f;
+    gs[to] = 1.f;
+  }
+  __syncthreads();
+  float* S = row + (size_t)h * D * V;
+  float s[DR_ROWS];
+  float d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+  for (int i = 0; i < DR_ROWS; ++i) {
+    const int r = seg * DR_ROWS + i;
+    s[i] = col_ok && r < D ? S[(size_t)r * V + col] : 0.f;
+    const float q = qs[seg * DR_PAD + i], k = ks[seg * DR_PAD + i];
+    s[i] *= gs[seg * DR_PAD + i];
+    d1 = fmaf(s[i], k, d1);
+    d2 = fmaf(s[i], q, d2);
+    d3 = fmaf(k, q, d3);
+  }
+  d1 = seg_sum<NSEG>(d1);
+  d2 = seg_sum<NSEG>(d2);
+  d3 = seg_sum<NSEG>(d3);
+  const float u = col_ok ? beta[t * H + h] * (vc[t * H * V + (size_t)h * V + col] - d1) : 0.f;
+#pragma unroll
+  for (int i = 0; i < DR_ROWS; ++i) {
+    const int r = seg * DR_ROWS + i;
+    if (col_ok && r < D) S[(size_t)r * V + col] = fmaf(ks[seg * DR_PAD + i], u, s[i]);
+  }
+  const float o = col_ok ? fmaf(u, d3, d2) : 0.f;
+  const float ss = block_sum(seg == 0 ? o * o : 0.f, red);
+  const float rs = 1.0f / sqrtf(ss / (float)V + eps);
+  if (col_ok && seg == 0)
+    out[t * H * V + (size_t)h * V + col] = from_f32<act_t>(o * rs * norm_w[col] * sigmoid_f(gate[col]));
+  // the convolution's inputs move on by this token: the head's own value channels, and its q/k head's if it is the first to read them
+  const int C = dd_channels(dm), NP = dd_np(dm);
+  float* hist = row + (size_t)H * D * V;
+  const bool first = h % (H / G) == 0;
+  const int mine = V + (first ? 2 * D : 0);
+  for (int i = tid; i < mine; i += blockDim.x) {
+    const int c = i < V ? 2 * G * D + h * V + i : (i - V < D ? gq * D + (i - V) : G * D + gq * D + (i - V - D));
+    float* hc = hist + (size_t)c * (K - 1);
+    for (int m = 0; m + 1 < K - 1; ++m) hc[m] = hc[m + 1];
+    if (K > 1) hc[K - 2] = P[t * NP + c];
+  }
+  (void)C;
+}
+
 // ------------------------------------------------------------------------------------------ entry points
 static int dims_ok(const DeltaDims& d) {
   return d.H > 0 && d.G > 0 && d.H % d.G == 0 && d.D > 0 && d.D <= 256 && d.V > 0 && d.taps >= 1 && d.taps <= 64 &&
@@ -449,6 +557,42 @@ TQ_API int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
   hipLaunchKernelGGL(delta_out_kernel, dim3(T + B, (H + 3) / 4 < 65535 ? (H + 3) / 4 : 65535), dim3(256), 0, st, o_raw, ag, norm_w, eps, P, cu_seqlens, slots, state,
                      state_stride, d, T, (act_t*)out);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// A decode step (one token per sequence, T == B) from delta_prep's outputs to the mixer's output `out` [T][H V]
+// (activation type), in one launch: returns TQ_ERR_UNSUPPORTED where a head's lanes do not fit one workgroup (the caller
+// then takes the kernels of longer steps).  low [T][ra + rg] (activation type); w_low [(H D + H V)][ra + rg] of wtype,
+// the block-diagonal matrix of both second low-rank products.
+TQ_API int tq_delta_decode(const float* qn, const float* kn, const float* vc, const float* beta, const void* low,
+                           const void* w_low, int wtype, const float* a_log, const float* dt_bias, const float* norm_w,
+                           float eps, const float* P, const int* cu_seqlens, const int* slots, float* state,
+                           int64_t state_stride, int H, int G, int D, int V, int taps, int ra, int rg, int B, void* out,
+                           hipStream_t st) {
+  if (B <= 0) return 0;
+  const DeltaDims d{H, G, D, V, taps, ra, rg};
+  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
+  int nseg = 1;
+  while (nseg * DR_ROWS < D) nseg *= 2;
+  const int threads = (nseg * V + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
+  if (threads > 1024 || B > 65535 || H > 65535) return TQ_ERR_UNSUPPORTED;
+  const size_t shmem = (size_t)(3 * DR_PAD * nseg + (V + 3) / 4 * 4 + (ra + rg + 3) / 4 * 4 + 16) * sizeof(float);
+  if (shmem > 60 * 1024) return TQ_ERR_UNSUPPORTED;
+#define TQ_DECODE(NS)                                                                                                 \
+  hipLaunchKernelGGL((delta_decode_kernel<NS, W>), dim3(H, B), dim3(threads), shmem, st, qn, kn, vc, beta,            \
+                     (const act_t*)low, (const W*)w_low, a_log, dt_bias, norm_w, eps, P, cu_seqlens, slots, state,    \
+                     state_stride, d, (act_t*)out)
+  TQ_DISPATCH_W(wtype, {
+    switch (nseg) {
+      case 1: TQ_DECODE(1); break;
+      case 2: TQ_DECODE(2); break;
+      case 4: TQ_DECODE(4); break;
+      case 8: TQ_DECODE(8); break;
+      default: TQ_DECODE(16); break;
+    }
+  });
+#undef TQ_DECODE
   TQ_LAUNCH_CHECK();
   return 0;
 }

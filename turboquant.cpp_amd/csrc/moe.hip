@@ -161,7 +161,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
   }
   if (groups > 1 && keep < groups) {
     const int per = E / groups;
-    // a lane per group (in turns of 64): the group's largest logit; then `keep` rounds choose the best groups
+    // a lane per group (in turns of 64): the group's largest logit
     float gmax[4];      // up to 256 groups
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -171,29 +171,26 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
         for (int e = gi * per; e < (gi + 1) * per; ++e) m = fmaxf(m, lg[e]);
       gmax[i] = m;
     }
+    // a group is kept if fewer than `keep` groups are better: a larger best logit, or the same and a higher index (the
+    // order in which rounds of a search would take them, without the rounds: every lane looks at every group once)
     unsigned kept = 0;      // bit i: group lane + 64 i is kept
-    for (int k = 0; k < keep; ++k) {
-      float bv = -INFINITY;
-      int bi = -1;
+    int better[4] = {0, 0, 0, 0};
+    for (int g2 = 0; g2 < groups; ++g2) {
+      const int src = g2 % 64;
+      float other = __shfl(gmax[0], src, TQ_WAVE);
+      if (groups > 64) {
+        const float o1 = __shfl(gmax[1], src, TQ_WAVE), o2 = __shfl(gmax[2], src, TQ_WAVE), o3 = __shfl(gmax[3], src, TQ_WAVE);
+        other = g2 < 64 ? other : g2 < 128 ? o1 : g2 < 192 ? o2 : o3;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int gi = lane + 64 * i;
-        if (gi < groups && !((kept >> i) & 1u) && gmax[i] >= bv) {
-          bv = gmax[i];
-          bi = gi;
-        }
+        better[i] += (other > gmax[i] || (other == gmax[i] && g2 > gi)) ? 1 : 0;
       }
-#pragma unroll
-      for (int o = TQ_WAVE / 2; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, TQ_WAVE);
-        const int oi = __shfl_xor(bi, o, TQ_WAVE);
-        if (oi >= 0 && (bi < 0 || ov > bv || (ov == bv && oi > bi))) {
-          bv = ov;
-          bi = oi;
-        }
-      }
-      if (bi >= 0 && bi % 64 == lane) kept |= 1u << (bi / 64);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (lane + 64 * i < groups && better[i] < keep) kept |= 1u << i;
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

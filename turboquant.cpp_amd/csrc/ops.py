@@ -71,6 +71,8 @@ _SIGNATURES = {
                       _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_delta_scan": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_delta_decode": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr,
+                        _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_delta_out": [_c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -187,7 +189,7 @@ _PROFILE: list | None = None
 _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pair": "matmul", "qkv_rope_write": "matmul",
          "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
          "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
-         "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn"}
+         "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn"}
 
 
 def profile_begin() -> None:
@@ -927,6 +929,10 @@ def _expert_groups(k: str, E: int, top_k: int, groups) -> tuple[int, int]:
     count, keep = int(groups[0]), int(groups[1])
     _need(1 <= count <= 256 and E % count == 0 and 1 <= keep <= count and top_k <= keep * (E // count), k,
           lambda: f"{count} groups of which {keep} are kept do not fit {E} experts with {top_k} per token")
+    if keep >= top_k or keep == count:
+        # nothing is ever left out: the best top_k experts lie in at most top_k groups, each of which has a better best
+        # expert than any group without one of them, so all of these groups are among the kept
+        return 1, 1
     return count, keep
 
 
@@ -1109,6 +1115,47 @@ def delta_out(o: torch.Tensor, ag: torch.Tensor, norm_w: torch.Tensor, eps: floa
     _run(k, library(act).tq_delta_out(_ptr(o), _ptr(ag), _ptr(norm_w), float(eps), _ptr(proj), _ptr(runs["cu_seqlens"]),
                                       _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), dims.rank_a, dims.rank_g, T,
                                       B, _ptr(out), _stream()))
+    return out
+
+
+def delta_decode_fits(dims: DeltaDims) -> bool:
+    """Whether a head's lanes (16 key channels of a value channel each) fit the one workgroup of ``delta_decode``."""
+    nseg = 1
+    while nseg * 16 < dims.dim:
+        nseg *= 2
+    return -(-nseg * dims.vdim // 64) * 64 <= 1024
+
+
+def delta_decode(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, low: torch.Tensor,
+                 low_weight: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                 proj: torch.Tensor, runs: dict, state: torch.Tensor, dims: DeltaDims, act) -> torch.Tensor:
+    """A decode step (one token per sequence) from ``delta_prep``'s outputs to the mixer's output [T, H*vdim] in the
+    activation type, in one launch: what the product over ``low_weight`` (the block-diagonal matrix of both second
+    low-rank products, [H*dim + H*vdim, rank_a + rank_g]), ``delta_scan`` and ``delta_out`` do in three (a row of that
+    product is summed by four lanes, each over every fourth element of the rank)."""
+    k = "delta_decode"
+    T = qn.shape[0]
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    R = dims.rank_a + dims.rank_g
+    for name, t, w in (("qn", qn, G * D), ("kn", kn, G * D), ("vc", vc, H * V), ("beta", beta, H)):
+        _check(t, k, name, torch.float32, (T, w))
+    _check(low, k, "low", ACT_DTYPES[dtype_name(act)], (T, R))
+    _check(low_weight, k, "low_weight", tuple(_WTYPE), (H * D + H * V, R))
+    _check(a_log, k, "a_log", torch.float32, (H,))
+    _check(dt_bias, k, "dt_bias", torch.float32, (H * D,))
+    _check(norm_w, k, "norm_w", torch.float32, (V,))
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    stride = _delta_state(k, state, dims)
+    B = runs["slots"].numel()
+    _need(T == B and runs["decode"], k, "a decode step brings one token per sequence")
+    _need(delta_decode_fits(dims), k, "a head's lanes do not fit one workgroup")
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    out = torch.empty((T, H * V), dtype=ACT_DTYPES[dtype_name(act)], device=qn.device)
+    _run(k, library(act).tq_delta_decode(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(low), _ptr(low_weight),
+                                         _WTYPE[low_weight.dtype], _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), float(eps),
+                                         _ptr(proj), _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride,
+                                         *dims.sizes(), dims.rank_a, dims.rank_g, B, _ptr(out), _stream()))
     return out
 
 

@@ -106,6 +106,10 @@ int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float
 int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w, float eps, const float* P,
         const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V,
         int taps, int ra, int rg, int T, int B, void* out, hipStream_t st);
+int tq_delta_decode(const float* qn, const float* kn, const float* vc, const float* beta, const void* low,
+        const void* w_low, int wtype, const float* a_log, const float* dt_bias, const float* norm_w, float eps,
+        const float* P, const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
+        int V, int taps, int ra, int rg, int B, void* out, hipStream_t st);
 // moe.hip: router, choice of experts, order of pairs (both libraries)
 int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
         int* ids, float* weights, float* shared_gate, float* logits, int T, int H, hipStream_t st);

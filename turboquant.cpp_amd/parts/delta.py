@@ -13,9 +13,10 @@ per value channel (shared by the heads) and by sigmoid(W_g2 (W_g1 x)), and the h
 
 The sequence's state is one row of float32 per slot (``StateNeed``): S, then the convolution's last taps - 1 inputs of
 every channel.  Decays, gates, norms and the recurrence are float32 on both libraries; the products are the
-activation type's.  Six launches a step, prompt or decode: the product of all first projections, ``delta_prep``, the
-second product of decay and gate (one product over a block-diagonal matrix of both), ``delta_scan`` (which, in a step
-of many tokens, first works out all decays in a launch of their own), ``delta_out``, the output product.
+activation type's.  Six launches a prompt step: the product of all first projections, ``delta_prep``, the second product
+of decay and gate (one product over a block-diagonal matrix of both), ``delta_scan`` (which, in a step of many tokens,
+first works out all decays in a launch of their own), ``delta_out``, the output product.  Four a decode step:
+``delta_decode`` stands for the three in the middle.
 """
 from __future__ import annotations
 
@@ -91,6 +92,11 @@ class ChannelDeltaRule(Part):
         runs = b.runs()
         proj = ops.gemm(normed, self.in_weight, ctx.act)
         qn, kn, vc, beta, low = ops.delta_prep(proj, b.slot_of_token, state, self.conv, d, ctx.act)
+        if b.is_decode and ops.delta_decode_fits(d):
+            # one token per sequence: second products, decays, recurrence, norm, gate and new convolution state in one launch
+            out = ops.delta_decode(qn, kn, vc, beta, low, self.low_weight, self.a_log, self.dt_bias, self.out_norm, self.eps,
+                                   proj, runs, state, d, ctx.act)
+            return ops.gemm(out, self.out_weight, ctx.act, partial_sums=True)
         ag = ops.gemm(low, self.low_weight, ctx.act)
         o = ops.delta_scan(qn, kn, vc, beta, ag, self.a_log, self.dt_bias, runs, state, d, ctx.act)
         out = ops.delta_out(o, ag, self.out_norm, self.eps, proj, runs, state, d, ctx.act)
