@@ -71,6 +71,7 @@ class ModelPlan:
     stop_tokens: tuple[int, ...] = ()
     embedding_scale: float = 1.0            # the embedding rows are multiplied by it
     logit_softcap: float | None = None      # logits <- cap * tanh(logits / cap)
+    logit_scale: float = 1.0                # the logits are multiplied by it, before the cap
     position_table: Source | None = None    # a learned vector per position [max_positions, H], added to the embedded token
 
     def validate(self) -> None:

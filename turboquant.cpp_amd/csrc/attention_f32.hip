@@ -164,6 +164,10 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
+  if (p.mod.sink) {         // a score without key or value, counted once
+    m_run = p.mod.sink[h];
+    l_run = 1.f;
+  }
 
   // what the block as a whole can reach, and what this wave can
   const int blk_first = start + blk * 64, blk_last = start + min(n_new, blk * 64 + 64) - 1;
@@ -327,6 +331,10 @@ __global__ __launch_bounds__(64) void attn_f32_join_kernel(AttnF32Args p) {
   for (int tile = first + lane; tile <= last; tile += 64) m = fmaxf(m, part[(size_t)tile * stride]);
   m = wave_max(m);
   float l = 0.f;
+  if (p.mod.sink) {         // the sink joins here, once, like one more tile with a sum of 1 and no values
+    m = fmaxf(m, p.mod.sink[h]);
+    l = expf(p.mod.sink[h] - m);
+  }
   for (int t0 = first; t0 <= last; t0 += 64) {
     const int tile = t0 + lane;
     float w = 0.f, wl = 0.f;
@@ -389,12 +397,12 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
 // The tokens are runs of consecutive positions, one per sequence (cu_seqlens, slots, start as in AttnF32Args);
 // decode: every run is one token and `partial` holds tq_attention_f32_scratch(B, nh, hd, max_end) floats.
 // hd must be a multiple of 4 and at most 256, page_size a multiple of 64, page_stride a multiple of 4.
-// softcap, r1, r2, chunk: see score_mod.h (0, null, null, 0: nothing).
+// softcap, r1, r2, chunk, sink: see score_mod.h (0, null, null, 0, null: nothing).
 TQ_API int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
                                 const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
                                 int B, int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1,
-                                const float* r2, int chunk, void* out, void* partial, int decode, int max_new,
-                                int max_end, hipStream_t st) {
+                                const float* r2, int chunk, const float* sink, void* out, void* partial, int decode,
+                                int max_new, int max_end, hipStream_t st) {
   if (B <= 0) return 0;
   if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
   if (hd <= 0 || hd % 4 != 0 || hd > 256 || nkv <= 0 || nh % nkv != 0 || page_size % AT != 0 || page_stride % 4 != 0)
@@ -404,7 +412,7 @@ TQ_API int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v
   if (max_new <= 0 || max_end <= 0) return TQ_ERR_BAD_ARG;
   AttnF32Args p{(const float*)q, (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, cu_seqlens, slots,
                 start, page_size, page_stride, nh, nkv, hd, window, scale, (float*)out, (float*)partial,
-                (max_end + AT - 1) / AT, ScoreMod{softcap, r1, r2, chunk}};
+                (max_end + AT - 1) / AT, ScoreMod{softcap, r1, r2, chunk, sink}};
   int rc;
   if (hd <= 16) rc = launch_attention_f32<1>(p, B, decode, max_new, max_end, st);
   else if (hd <= 32) rc = launch_attention_f32<2>(p, B, decode, max_new, max_end, st);
@@ -421,6 +429,6 @@ TQ_API int tq_attention_f32(const void* q, const void* k_pool, const void* v_poo
                             int B, int nh, int nkv, int hd, int window, float scale, void* out, void* partial, int decode,
                             int max_new, int max_end, hipStream_t st) {
   return tq_attention_f32_mod(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride,
-                              B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, partial, decode, max_new,
+                              B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, nullptr, out, partial, decode, max_new,
                               max_end, st);
 }

@@ -40,6 +40,10 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
   // each thread owns the output dimensions tid, tid + CHUNK, ... (at most 4: hd <= 512)
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
+  if (mod.sink) {        // a score without key or value, counted once
+    m_run = mod.sink[h];
+    l_run = 1.f;
+  }
 
   for (int base = (lo / CHUNK) * CHUNK; base <= pos; base += CHUNK) {
     const int j = base + tid;
@@ -88,16 +92,16 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
   }
 }
 
-// softcap, r1, r2, chunk: what happens to a score before the softmax and the chunks of positions, see score_mod.h
-// (0, null, null, 0: nothing).
+// softcap, r1, r2, chunk, sink: what happens to a score before the softmax and the chunks of positions, see score_mod.h
+// (0, null, null, 0, null: nothing).
 TQ_API int tq_attention_generic_mod(const void* q, const void* k_pool, const void* v_pool, const int* positions,
                                     const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
                                     int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
-                                    float softcap, const float* r1, const float* r2, int chunk, void* out,
-                                    hipStream_t st) {
+                                    float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                    void* out, hipStream_t st) {
   if (T <= 0) return 0;
   if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
-  const ScoreMod mod{softcap, r1, r2, chunk};
+  const ScoreMod mod{softcap, r1, r2, chunk, sink};
   if (hd > 4 * CHUNK || nkv <= 0 || nh % nkv != 0) return TQ_ERR_UNSUPPORTED;
   if (nh > 65535) return TQ_ERR_UNSUPPORTED;
   const size_t shmem = (size_t)(hd + CHUNK + 4) * sizeof(float) + CHUNK * (sizeof(int64_t) + sizeof(int));
@@ -113,5 +117,5 @@ TQ_API int tq_attention_generic(const void* q, const void* k_pool, const void* v
                                 int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
                                 void* out, hipStream_t st) {
   return tq_attention_generic_mod(q, k_pool, v_pool, positions, seq_of_token, block_table, bt_stride, page_size,
-                                  page_stride, T, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, st);
+                                  page_stride, T, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, nullptr, out, st);
 }

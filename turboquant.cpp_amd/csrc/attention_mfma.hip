@@ -461,6 +461,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int dt = 0; dt < DT; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     m_run[g] = -INFINITY;
     l_run[g] = 0.f;
+    if (a.mod.sink) {       // a score without key or value, counted once; maxima are in units of log2
+      m_run[g] = a.mod.sink[h] * LOG2E;
+      l_run[g] = 1.f;
+    }
   }
   // tiles the workgroup goes through, and those among them that this wave's tokens can see
   const int wg_first = start + qb, wg_last = start + min(qb + 4 * QW, n) - 1;
@@ -623,6 +627,10 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
   for (int s = run_beg + lane; s < run_end; s += 64) m = fmaxf(m, part[(size_t)s * stride + a.hd]);
   m = wave_max(m);
   float l = 0.f;
+  if (a.mod.sink) {         // the sink joins here, once, like one more run with a sum of 1 and no values
+    m = fmaxf(m, a.mod.sink[h] * LOG2E);
+    l = __builtin_amdgcn_exp2f(a.mod.sink[h] * LOG2E - m);
+  }
   for (int s0 = run_beg; s0 < run_end; s0 += 64) {     // denominators in run order, 64 runs at a time
     const int s = s0 + lane;
     float w = 0.f, wl = 0.f;
@@ -697,12 +705,12 @@ TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
 
 // decode != 0: every sequence brings exactly one token.  max_new: longest run of new tokens of a sequence;
 // max_end: largest position + 1 that any token of the step has.
-// softcap, r1, r2, chunk: see score_mod.h (0, null, null, 0: nothing).
+// softcap, r1, r2, chunk, sink: see score_mod.h (0, null, null, 0, null: nothing).
 TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                                  int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
                                  int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
-                                 float softcap, const float* r1, const float* r2, int chunk, void* out,
-                                 float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+                                 float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                 void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st) {
   if (B <= 0) return 0;
   if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
   if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
@@ -711,7 +719,7 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
   if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
-             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk}};
+             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk, sink}};
   const int dt = hd / 16;
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
@@ -745,6 +753,6 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
                              int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale, void* out,
                              float* partial, int decode, int max_new, int max_end, hipStream_t st) {
   return tq_attention_mfma_mod(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride,
-                               B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, out, partial, decode, max_new,
+                               B, nh, nkv, hd, window, scale, 0.f, nullptr, nullptr, 0, nullptr, out, partial, decode, max_new,
                                max_end, st);
 }

@@ -18,6 +18,10 @@
 //   delta_decode (steps of one token per sequence) the second low-rank products, decays, recurrence, norm, gate and the
 //                convolution's new state in one launch
 //
+// A second form (DeltaDims.mode 1) has one decay per head, g = exp(-exp(A_log_h) * softplus(a_h + dt_bias_h)) with a_h a
+// projection of its own, and a gate that is a full projection with an activation of the caller's choice (gates.def); its
+// projections are q | k | v | b (H) | a (H) | gate (H V), and it has no low-rank products.  The same kernels serve it.
+//
 // A sequence's row of state (float): S as [H][D][V], then for every convolution channel (q's, k's, v's) its last
 // taps - 1 inputs, oldest first.  Projections P [T][NP] (float): q (G D) | k (G D) | v (H V) | b (H) | a1 (ra) | g1 (rg).
 #include "common.h"
@@ -29,9 +33,12 @@ struct DeltaDims {
   int H, G, D, V;         // heads, q/k heads, key width, value width
   int taps;               // of the convolution
   int ra, rg;             // ranks of the decay's and the gate's first product
+  int mode;               // 0: a decay per head and key channel, behind low-rank products; 1: a decay per head (ra = rg = 0)
 };
 __host__ __device__ __forceinline__ int dd_channels(const DeltaDims& d) { return 2 * d.G * d.D + d.H * d.V; }
-__host__ __device__ __forceinline__ int dd_np(const DeltaDims& d) { return dd_channels(d) + d.H + d.ra + d.rg; }
+__host__ __device__ __forceinline__ int dd_np(const DeltaDims& d) {
+  return d.mode == 1 ? dd_channels(d) + 2 * d.H + d.H * d.V : dd_channels(d) + d.H + d.ra + d.rg;
+}
 __host__ __device__ __forceinline__ int64_t dd_state(const DeltaDims& d) {
   return (int64_t)d.H * d.D * d.V + (int64_t)dd_channels(d) * (d.taps - 1);
 }
@@ -50,7 +57,8 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict
                                                          const float* __restrict__ conv_w, DeltaDims dm,
                                                          float* __restrict__ qn, float* __restrict__ kn,
                                                          float* __restrict__ vc, float* __restrict__ beta,
-                                                         act_t* __restrict__ low) {
+                                                         act_t* __restrict__ low, const float* __restrict__ a_log,
+                                                         const float* __restrict__ dt_bias, float* __restrict__ dec) {
   const int t = blockIdx.x, wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   const int G = dm.G, D = dm.D, H = dm.H, V = dm.V, K = dm.taps;
   const int NP = dd_np(dm), C = dd_channels(dm);
@@ -63,6 +71,11 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict
   for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
     if (u == units - 1) {
       for (int h = lane; h < H; h += TQ_WAVE) beta[(size_t)t * H + h] = sigmoid_f(row[C + h]);
+      if (dm.mode == 1) {       // the decay of every head
+        for (int h = lane; h < H; h += TQ_WAVE)
+          dec[(size_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(row[C + H + h] + dt_bias[h]));
+        continue;
+      }
       for (int i = lane; i < dm.ra + dm.rg; i += TQ_WAVE)
         low[(size_t)t * (dm.ra + dm.rg) + i] = from_f32<act_t>(row[C + H + i]);
       continue;
@@ -141,7 +154,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
                                                          const float* __restrict__ dt_bias,
                                                          const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
                                                          float* __restrict__ state, int64_t state_stride, DeltaDims dm,
-                                                         int cols, int col_blocks, float* __restrict__ o_raw) {
+                                                         int cols, int col_blocks, int head_decay,
+                                                         float* __restrict__ o_raw) {
   constexpr int DP = DR_ROWS * NSEG, RL = DR_PAD * NSEG;      // rows of a token, and the floats they take in LDS
   constexpr int EV = 16 * CPT / NSEG > 0 ? 16 * CPT / NSEG : 1;      // values of v per thread and chunk, at the most
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -185,7 +199,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
       const size_t t = (size_t)(t0 + c0 + c);
       rq[j] = qn[t * G * D + (size_t)gq * D + r];
       rk[j] = kn[t * G * D + (size_t)gq * D + r];
-      rg[j] = ag[t * AGW + (size_t)h * D + r];
+      rg[j] = head_decay ? ag[t * H + h] : ag[t * AGW + (size_t)h * D + r];      // (head_decay: ag is [T][H] decays)
     }
 #pragma unroll
     for (int j = 0; j < EV; ++j) {
@@ -303,10 +317,11 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
 }
 
 // ------------------------------------------------------------------------------------------ norm, gate, new inputs
-// grid (T + B, Y), block 256.  Blocks 0 .. T - 1 of x: a wave per head of its token: o / rms(o) * w * sigmoid(gate).
+// grid (T + B, Y), block 256.  Blocks 0 .. T - 1 of x: a wave per head of its token: o / rms(o) * w * f(gate), the gate's row of token t at gates + t * gate_ld, f an activation of gates.def.
 // Blocks T ..: the convolution's state of one sequence, its channels dealt over y: its last taps - 1 inputs, those of this run and, where the run
 // is shorter, the most recent of the old state before them.
-__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const float* __restrict__ ag,
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const float* __restrict__ gates,
+                                                        int64_t gate_ld, int gate_kind,
                                                         const float* __restrict__ norm_w, float eps,
                                                         const float* __restrict__ P, const int* __restrict__ cu_seqlens,
                                                         const int* __restrict__ slots, float* __restrict__ state,
@@ -315,16 +330,15 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
   const int H = dm.H, D = dm.D, V = dm.V, K = dm.taps;
   if ((int)blockIdx.x < T) {
     const int t = blockIdx.x, wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
-    const int AGW = H * D + H * V;
     for (int h = blockIdx.y * 4 + wave; h < H; h += 4 * gridDim.y) {
       const float* o = o_raw + (size_t)t * H * V + (size_t)h * V;
       float ss = 0.f;
       for (int j = lane; j < V; j += TQ_WAVE) ss += o[j] * o[j];
       ss = wave_sum(ss);
       const float rs = 1.0f / sqrtf(ss / (float)V + eps);
-      const float* gate = ag + (size_t)t * AGW + (size_t)H * D + (size_t)h * V;
+      const float* gate = gates + (size_t)t * gate_ld + (size_t)h * V;
       for (int j = lane; j < V; j += TQ_WAVE)
-        out[(size_t)t * H * V + (size_t)h * V + j] = from_f32<act_t>(o[j] * rs * norm_w[j] * sigmoid_f(gate[j]));
+        out[(size_t)t * H * V + (size_t)h * V + j] = from_f32<act_t>(o[j] * rs * norm_w[j] * gate_fn(gate[j], gate_kind));
     }
     return;
   }
@@ -358,7 +372,8 @@ __global__ __launch_bounds__(1024) void delta_decode_kernel(const float* __restr
                                                             const float* __restrict__ norm_w, float eps,
                                                             const float* __restrict__ P, const int* __restrict__ cu_seqlens,
                                                             const int* __restrict__ slots, float* __restrict__ state,
-                                                            int64_t state_stride, DeltaDims dm, act_t* __restrict__ out) {
+                                                            int64_t state_stride, DeltaDims dm, int gate_kind,
+                                                            act_t* __restrict__ out) {
   constexpr int DP = DR_ROWS * NSEG, RL = DR_PAD * NSEG;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                 // [RL] each: a lane's 16 rows 20 floats from its neighbour's
@@ -373,13 +388,28 @@ __global__ __launch_bounds__(1024) void delta_decode_kernel(const float* __restr
   const bool col_ok = col < V;
   const size_t t = (size_t)cu_seqlens[b];
   float* row = state + (size_t)slots[b] * state_stride;
-  for (int i = tid; i < R; i += blockDim.x) lowv[i] = to_f32(low[t * R + i]);
+  for (int i = tid; i < R; i += blockDim.x) lowv[i] = to_f32(low[t * R + i]);       // (mode 1: R is 0)
   __syncthreads();
   const float rate = expf(a_log[h]);
   // The head's D rows of the decay's product and V rows of the gate's, four neighbouring lanes to a row: lane p of the
   // four sums the elements p, p + 4, ... of the rank, and the four partial sums are added within the quad.
   const int part = tid & 3, rows_a_pass = (int)blockDim.x >> 2;
-  for (int r0 = 0; r0 < D + V; r0 += rows_a_pass) {
+  if (dm.mode == 1) {
+    // a decay per head and a gate that is a projection of its own: nothing to multiply here
+    const int C1 = dd_channels(dm), NP1 = dd_np(dm);
+    const float g = expf(-rate * softplus_f(P[t * NP1 + C1 + H + h] + dt_bias[h]));
+    for (int r = tid; r < D + V; r += blockDim.x) {
+      if (r < D) {
+        const int to = r / DR_ROWS * DR_PAD + r % DR_ROWS;
+        qs[to] = qn[t * G * D + (size_t)gq * D + r];
+        ks[to] = kn[t * G * D + (size_t)gq * D + r];
+        gs[to] = g;
+      } else {
+        gate[r - D] = P[t * NP1 + C1 + 2 * H + (size_t)h * V + (r - D)];
+      }
+    }
+  }
+  for (int r0 = 0; dm.mode == 0 && r0 < D + V; r0 += rows_a_pass) {
     const int r = r0 + (tid >> 2);
     const bool live = r < D + V, decay = r < D;
     float a = 0.f;
@@ -434,7 +464,7 @@ __global__ __launch_bounds__(1024) void delta_decode_kernel(const float* __restr
   const float ss = block_sum(seg == 0 ? o * o : 0.f, red);
   const float rs = 1.0f / sqrtf(ss / (float)V + eps);
   if (col_ok && seg == 0)
-    out[t * H * V + (size_t)h * V + col] = from_f32<act_t>(o * rs * norm_w[col] * sigmoid_f(gate[col]));
+    out[t * H * V + (size_t)h * V + col] = from_f32<act_t>(o * rs * norm_w[col] * gate_fn(gate[col], gate_kind));
   // the convolution's inputs move on by this token: the head's own value channels, and its q/k head's if it is the first to read them
   const int C = dd_channels(dm), NP = dd_np(dm);
   float* hist = row + (size_t)H * D * V;
@@ -452,13 +482,25 @@ __global__ __launch_bounds__(1024) void delta_decode_kernel(const float* __restr
 // ------------------------------------------------------------------------------------------ entry points
 static int dims_ok(const DeltaDims& d) {
   return d.H > 0 && d.G > 0 && d.H % d.G == 0 && d.D > 0 && d.D <= 256 && d.V > 0 && d.taps >= 1 && d.taps <= 64 &&
-         d.ra > 0 && d.rg > 0;
+         (d.mode == 1 ? d.ra == 0 && d.rg == 0 : d.mode == 0 && d.ra > 0 && d.rg > 0);
 }
 
 // Floats of one sequence's row of state.
 TQ_API int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps) {
-  const DeltaDims d{H, G, D, V, taps, 1, 1};
+  const DeltaDims d{H, G, D, V, taps, 1, 1, 0};
   return dd_state(d);
+}
+
+static int launch_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
+                       const float* conv_w, const DeltaDims& d, float* qn, float* kn, float* vc, float* beta, void* low,
+                       const float* a_log, const float* dt_bias, float* dec, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
+  const int units = 2 * d.G + d.H + 1;
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(T, (units + 3) / 4 < 65535 ? (units + 3) / 4 : 65535), dim3(256), 0, st, P,
+                     slot_of_token, state, state_stride, conv_w, d, qn, kn, vc, beta, (act_t*)low, a_log, dt_bias, dec);
+  TQ_LAUNCH_CHECK();
+  return 0;
 }
 
 // P [T][NP] float (see the head of this file); slot_of_token [T]; state: rows of state_stride floats by slot;
@@ -467,27 +509,28 @@ TQ_API int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps) {
 TQ_API int tq_delta_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
                          const float* conv_w, int H, int G, int D, int V, int taps, int ra, int rg, float* qn, float* kn,
                          float* vc, float* beta, void* low, int T, hipStream_t st) {
-  if (T <= 0) return 0;
-  const DeltaDims d{H, G, D, V, taps, ra, rg};
-  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
-  const int units = 2 * G + H + 1;
-  hipLaunchKernelGGL(delta_prep_kernel, dim3(T, (units + 3) / 4 < 65535 ? (units + 3) / 4 : 65535), dim3(256), 0, st, P, slot_of_token, state, state_stride, conv_w, d, qn,
-                     kn, vc, beta, (act_t*)low);
-  TQ_LAUNCH_CHECK();
-  return 0;
+  return launch_prep(P, slot_of_token, state, state_stride, conv_w, DeltaDims{H, G, D, V, taps, ra, rg, 0}, qn, kn, vc, beta,
+                     low, nullptr, nullptr, nullptr, T, st);
 }
 
-// The recurrence over runs of tokens, one run per sequence (cu_seqlens [B + 1], slots [B], T tokens in all); the state
-// rows are read and written.  o_raw [T][H V] float.  In a step of many tokens the first H D columns of ag are replaced
-// by the decays they stand for (nothing else reads them afterwards).
-TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, float* ag,
-                         const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
-                         int64_t state_stride, int H, int G, int D, int V, int taps, int T, int B, float* o_raw,
-                         hipStream_t st) {
+// The form with a decay per head: P [T][q | k | v | b (H) | a (H) | gate (H V)]; writes qn, kn, vc, beta as above and
+// dec [T][H] = exp(-exp(a_log[h]) * softplus(a + dt_bias[h])).
+TQ_API int tq_delta_prep_h(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
+                           const float* conv_w, const float* a_log, const float* dt_bias, int H, int G, int D, int V,
+                           int taps, float* qn, float* kn, float* vc, float* beta, float* dec, int T, hipStream_t st) {
+  if (!a_log || !dt_bias || !dec) return TQ_ERR_BAD_ARG;
+  return launch_prep(P, slot_of_token, state, state_stride, conv_w, DeltaDims{H, G, D, V, taps, 0, 0, 1}, qn, kn, vc, beta,
+                     nullptr, a_log, dt_bias, dec, T, st);
+}
+
+// head_decay: ag is [T][H], the decay of every head, ready to use.
+static int launch_scan(const float* qn, const float* kn, const float* vc, const float* beta, float* ag, const float* a_log,
+                       const float* dt_bias, const int* cu_seqlens, const int* slots, float* state, int64_t state_stride,
+                       const DeltaDims& d, int head_decay, int T, int B, float* o_raw, hipStream_t st) {
   if (B <= 0 || T <= 0) return 0;
-  const DeltaDims d{H, G, D, V, taps, 1, 1};
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
   if (B > 65535) return TQ_ERR_UNSUPPORTED;
+  const int H = d.H, D = d.D, V = d.V;
   int nseg = 1;
   while (nseg * DR_ROWS < D) nseg *= 2;
   // value channels per lane: as many of 4, 2, 1 as still leave the head's lanes a whole wave
@@ -507,8 +550,8 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
   const int chunk = DR_CHUNK < DR_STAGE * threads / dp ? DR_CHUNK : DR_STAGE * threads / dp;
   const size_t shmem = (size_t)2 * (3 * chunk * DR_PAD * nseg + (chunk * cols + 3) / 4 * 4 + DR_CHUNK) * sizeof(float);
   // the decays of a long step are worked out beforehand, once for all blocks of value channels
-  const int decayed = T > 16 * B || T >= 256;
-  if (decayed) {
+  const int decayed = head_decay || T > 16 * B || T >= 256;
+  if (decayed && !head_decay) {
     const int64_t total = (int64_t)T * H * D;
     hipLaunchKernelGGL(delta_decay_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ag, a_log, dt_bias,
                        H * D, D, H * D + H * V, total);
@@ -520,7 +563,7 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                              \
     hipLaunchKernelGGL((delta_scan_kernel<NS, CP, DEC>), dim3(H * col_blocks, B), dim3(threads), shmem, st, qn, kn,   \
                        vc, beta, ag, a_log, dt_bias, cu_seqlens, slots, state, state_stride, d, cols, col_blocks,     \
-                       o_raw);                                                                                        \
+                       head_decay, o_raw);                                                                            \
   } while (0)
 #define TQ_SCAN_AS(NS, CP)                   \
   do {                                       \
@@ -547,17 +590,77 @@ TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, cons
   return 0;
 }
 
+// The recurrence over runs of tokens, one run per sequence (cu_seqlens [B + 1], slots [B], T tokens in all); the state
+// rows are read and written.  o_raw [T][H V] float.  In a step of many tokens the first H D columns of ag are replaced
+// by the decays they stand for (nothing else reads them afterwards).
+TQ_API int tq_delta_scan(const float* qn, const float* kn, const float* vc, const float* beta, float* ag,
+                         const float* a_log, const float* dt_bias, const int* cu_seqlens, const int* slots, float* state,
+                         int64_t state_stride, int H, int G, int D, int V, int taps, int T, int B, float* o_raw,
+                         hipStream_t st) {
+  return launch_scan(qn, kn, vc, beta, ag, a_log, dt_bias, cu_seqlens, slots, state, state_stride,
+                     DeltaDims{H, G, D, V, taps, 1, 1, 0}, 0, T, B, o_raw, st);
+}
+
+// The same recurrence with one decay per head: dec [T][H] as tq_delta_prep_h wrote it.
+TQ_API int tq_delta_scan_h(const float* qn, const float* kn, const float* vc, const float* beta, const float* dec,
+                           const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
+                           int V, int taps, int T, int B, float* o_raw, hipStream_t st) {
+  return launch_scan(qn, kn, vc, beta, const_cast<float*>(dec), nullptr, nullptr, cu_seqlens, slots, state, state_stride,
+                     DeltaDims{H, G, D, V, taps, 0, 0, 1}, 1, T, B, o_raw, st);
+}
+
+static int launch_out(const float* o_raw, const float* gates, int64_t gate_ld, int gate_kind, const float* norm_w, float eps,
+                      const float* P, const int* cu_seqlens, const int* slots, float* state, int64_t state_stride,
+                      const DeltaDims& d, int T, int B, void* out, hipStream_t st) {
+  if (T <= 0 || B <= 0) return 0;
+  if (!dims_ok(d) || state_stride < dd_state(d) || gate_kind < 0 || gate_kind >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(delta_out_kernel, dim3(T + B, (d.H + 3) / 4 < 65535 ? (d.H + 3) / 4 : 65535), dim3(256), 0, st, o_raw,
+                     gates, gate_ld, gate_kind, norm_w, eps, P, cu_seqlens, slots, state, state_stride, d, T, (act_t*)out);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // Norm and gate of every head's read-out into `out` [T][H V] (activation type), and every sequence's new convolution
-// state from P.  norm_w [V] float.
+// state from P.  norm_w [V] float.  The gate is the sigmoid of the last H V columns of ag.
 TQ_API int tq_delta_out(const float* o_raw, const float* ag, const float* norm_w, float eps, const float* P,
                         const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
                         int V, int taps, int ra, int rg, int T, int B, void* out, hipStream_t st) {
-  if (T <= 0 || B <= 0) return 0;
-  const DeltaDims d{H, G, D, V, taps, ra, rg};
-  if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
-  hipLaunchKernelGGL(delta_out_kernel, dim3(T + B, (H + 3) / 4 < 65535 ? (H + 3) / 4 : 65535), dim3(256), 0, st, o_raw, ag, norm_w, eps, P, cu_seqlens, slots, state,
-                     state_stride, d, T, (act_t*)out);
-  TQ_LAUNCH_CHECK();
+  return launch_out(o_raw, ag + (size_t)H * D, (int64_t)H * D + (int64_t)H * V, TQ_GATE_sigmoid, norm_w, eps, P, cu_seqlens,
+                    slots, state, state_stride, DeltaDims{H, G, D, V, taps, ra, rg, 0}, T, B, out, st);
+}
+
+// The form with a decay per head: the gate is activation `gate_kind` (gates.def) of the last H V columns of P.
+TQ_API int tq_delta_out_h(const float* o_raw, const float* norm_w, float eps, const float* P, int gate_kind,
+                          const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
+                          int V, int taps, int T, int B, void* out, hipStream_t st) {
+  const DeltaDims d{H, G, D, V, taps, 0, 0, 1};
+  return launch_out(o_raw, P + dd_channels(d) + 2 * H, dd_np(d), gate_kind, norm_w, eps, P, cu_seqlens, slots, state,
+                    state_stride, d, T, B, out, st);
+}
+
+template <class W>
+static int launch_decode(const float* qn, const float* kn, const float* vc, const float* beta, const void* low,
+                         const void* w_low, const float* a_log, const float* dt_bias, const float* norm_w, float eps,
+                         const float* P, const int* cu_seqlens, const int* slots, float* state, int64_t state_stride,
+                         const DeltaDims& d, int gate_kind, int B, void* out, hipStream_t st) {
+  int nseg = 1;
+  while (nseg * DR_ROWS < d.D) nseg *= 2;
+  const int threads = (nseg * d.V + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
+  if (threads > 1024 || B > 65535 || d.H > 65535) return TQ_ERR_UNSUPPORTED;
+  const size_t shmem = (size_t)(3 * DR_PAD * nseg + (d.V + 3) / 4 * 4 + (d.ra + d.rg + 3) / 4 * 4 + 16) * sizeof(float);
+  if (shmem > 60 * 1024) return TQ_ERR_UNSUPPORTED;
+#define TQ_DECODE(NS)                                                                                                 \
+  hipLaunchKernelGGL((delta_decode_kernel<NS, W>), dim3(d.H, B), dim3(threads), shmem, st, qn, kn, vc, beta,          \
+                     (const act_t*)low, (const W*)w_low, a_log, dt_bias, norm_w, eps, P, cu_seqlens, slots, state,    \
+                     state_stride, d, gate_kind, (act_t*)out)
+  switch (nseg) {
+    case 1: TQ_DECODE(1); break;
+    case 2: TQ_DECODE(2); break;
+    case 4: TQ_DECODE(4); break;
+    case 8: TQ_DECODE(8); break;
+    default: TQ_DECODE(16); break;
+  }
+#undef TQ_DECODE
   return 0;
 }
 
@@ -571,28 +674,29 @@ TQ_API int tq_delta_decode(const float* qn, const float* kn, const float* vc, co
                            int64_t state_stride, int H, int G, int D, int V, int taps, int ra, int rg, int B, void* out,
                            hipStream_t st) {
   if (B <= 0) return 0;
-  const DeltaDims d{H, G, D, V, taps, ra, rg};
+  const DeltaDims d{H, G, D, V, taps, ra, rg, 0};
   if (!dims_ok(d) || state_stride < dd_state(d)) return TQ_ERR_BAD_ARG;
-  int nseg = 1;
-  while (nseg * DR_ROWS < D) nseg *= 2;
-  const int threads = (nseg * V + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;
-  if (threads > 1024 || B > 65535 || H > 65535) return TQ_ERR_UNSUPPORTED;
-  const size_t shmem = (size_t)(3 * DR_PAD * nseg + (V + 3) / 4 * 4 + (ra + rg + 3) / 4 * 4 + 16) * sizeof(float);
-  if (shmem > 60 * 1024) return TQ_ERR_UNSUPPORTED;
-#define TQ_DECODE(NS)                                                                                                 \
-  hipLaunchKernelGGL((delta_decode_kernel<NS, W>), dim3(H, B), dim3(threads), shmem, st, qn, kn, vc, beta,            \
-                     (const act_t*)low, (const W*)w_low, a_log, dt_bias, norm_w, eps, P, cu_seqlens, slots, state,    \
-                     state_stride, d, (act_t*)out)
   TQ_DISPATCH_W(wtype, {
-    switch (nseg) {
-      case 1: TQ_DECODE(1); break;
-      case 2: TQ_DECODE(2); break;
-      case 4: TQ_DECODE(4); break;
-      case 8: TQ_DECODE(8); break;
-      default: TQ_DECODE(16); break;
-    }
+    const int rc = launch_decode<W>(qn, kn, vc, beta, low, w_low, a_log, dt_bias, norm_w, eps, P, cu_seqlens, slots, state,
+                                    state_stride, d, TQ_GATE_sigmoid, B, out, st);
+    if (rc) return rc;
   });
-#undef TQ_DECODE
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// The form with a decay per head and a gate of activation `gate_kind` that is a projection of its own (P as for
+// tq_delta_prep_h): the decay, the recurrence for the one token, norm, gate and the convolution's new state.
+TQ_API int tq_delta_decode_h(const float* qn, const float* kn, const float* vc, const float* beta, const float* a_log,
+                             const float* dt_bias, const float* norm_w, float eps, const float* P, int gate_kind,
+                             const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G,
+                             int D, int V, int taps, int B, void* out, hipStream_t st) {
+  if (B <= 0) return 0;
+  const DeltaDims d{H, G, D, V, taps, 0, 0, 1};
+  if (!dims_ok(d) || state_stride < dd_state(d) || gate_kind < 0 || gate_kind >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
+  const int rc = launch_decode<float>(qn, kn, vc, beta, nullptr, nullptr, a_log, dt_bias, norm_w, eps, P, cu_seqlens, slots,
+                                      state, state_stride, d, gate_kind, B, out, st);
+  if (rc) return rc;
   TQ_LAUNCH_CHECK();
   return 0;
 }

@@ -34,6 +34,22 @@ __global__ void softcap_kernel(float* __restrict__ x, int64_t n, float cap) {
   if (i < n) x[i] = cap * tanhf(x[i] / cap);
 }
 
+// x <- x * scale, then (cap > 0) x <- cap * tanh(x / cap): logits that a model multiplies by a constant before it caps them.
+__global__ void scale_softcap_kernel(float* __restrict__ x, int64_t n, float scale, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = x[i] * scale;
+  x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
+TQ_API int tq_scale_softcap(float* x, int64_t n, float scale, float cap, hipStream_t st) {
+  if (n <= 0) return 0;
+  if (cap < 0.f) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(scale_softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, n, scale, cap);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 TQ_API int tq_softcap(float* x, int64_t n, float cap, hipStream_t st) {
   if (n <= 0) return 0;
   if (!(cap > 0.f)) return TQ_ERR_BAD_ARG;
@@ -232,32 +248,93 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
 // ---------------------------------------------------------------- the gate of a gated pair, applied afterwards
 // out[m][n] = f(gu[m][n]) * gu[m][N + n]: for a pair of products that came out of one plain product over the two
 // matrices laid one behind the other (a library's, which has no such epilogue).  gu is float32 with row stride ld.
+// (the general form: the gate's rows at g with stride ldg, the other factor's at u with stride ldu; u null: out = f(g)
+// alone, an activation behind a plain product; gate < 0: f is the identity, a change of type)
 template <bool VEC>
-__global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gu, int64_t ld, act_t* __restrict__ out,
-                                                        int N, int gate) {
-  const float* row = gu + (size_t)blockIdx.y * ld;
+__global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gp, int64_t ldg, const float* __restrict__ up,
+                                                        int64_t ldu, act_t* __restrict__ out, int N, int gate) {
+  const float* row = gp + (size_t)blockIdx.y * ldg;
+  const float* urow = up ? up + (size_t)blockIdx.y * ldu : nullptr;
   act_t* dst = out + (size_t)blockIdx.y * N;
   if (VEC) {
     const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (n >= N) return;
-    const f32x4 g = load4f(row + n), u = load4f(row + N + n);
-    store4(dst + n, f32x4{gate_fn(g.x, gate) * u.x, gate_fn(g.y, gate) * u.y, gate_fn(g.z, gate) * u.z,
-                          gate_fn(g.w, gate) * u.w});
+    f32x4 g = load4f(row + n);
+    if (gate >= 0) g = f32x4{gate_fn(g.x, gate), gate_fn(g.y, gate), gate_fn(g.z, gate), gate_fn(g.w, gate)};
+    if (urow) g *= load4f(urow + n);
+    store4(dst + n, g);
   } else {
     const int n = blockIdx.x * 256 + threadIdx.x;
-    if (n < N) dst[n] = from_f32<act_t>(gate_fn(row[n], gate) * row[N + n]);
+    if (n >= N) return;
+    float g = row[n];
+    if (gate >= 0) g = gate_fn(g, gate);
+    if (urow) g *= urow[n];
+    dst[n] = from_f32<act_t>(g);
   }
 }
 
-TQ_API int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st) {
+static int launch_gated_act(const float* g, int64_t ldg, const float* u, int64_t ldu, void* out, int M, int N, int gate,
+                            hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
-  if (gate < 0 || gate >= TQ_GATE_COUNT || ld < 2 * (int64_t)N) return TQ_ERR_BAD_ARG;
+  if (gate >= TQ_GATE_COUNT || ldg < N || (u && ldu < N)) return TQ_ERR_BAD_ARG;
   if (M > 65535) return TQ_ERR_UNSUPPORTED;
-  const bool vec = N % 4 == 0 && ld % 4 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const bool vec = N % 4 == 0 && ldg % 4 == 0 && ((uintptr_t)g % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                   (!u || (ldu % 4 == 0 && ((uintptr_t)u % 16) == 0));
   if (vec)
-    hipLaunchKernelGGL(gated_act_kernel<true>, dim3((N / 4 + 255) / 256, M), dim3(256), 0, st, gu, ld, (act_t*)out, N, gate);
+    hipLaunchKernelGGL(gated_act_kernel<true>, dim3((N / 4 + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate);
   else
-    hipLaunchKernelGGL(gated_act_kernel<false>, dim3((N + 255) / 256, M), dim3(256), 0, st, gu, ld, (act_t*)out, N, gate);
+    hipLaunchKernelGGL(gated_act_kernel<false>, dim3((N + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+TQ_API int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st) {
+  if (gate < 0 || ld < 2 * (int64_t)N) return TQ_ERR_BAD_ARG;
+  return launch_gated_act(gu, ld, gu + N, ld, out, M, N, gate, st);
+}
+
+// out[m][n] = f(g[m][n]) * u[m][n] in the activation type, with rows of g and u at strides of their own; u null:
+// f(g) alone; gate < 0: no activation (with u null: the rows of g in the activation type).
+TQ_API int tq_act_rows(const float* g, int64_t ldg, const float* u, int64_t ldu, void* out, int M, int N, int gate,
+                       hipStream_t st) {
+  for (int r = 0; r < M; r += 65535) {          // the grid's y takes 65,535 rows at a time
+    const int rows = M - r < 65535 ? M - r : 65535;
+    const int rc = launch_gated_act(g + (size_t)r * ldg, ldg, u ? u + (size_t)r * ldu : nullptr, ldu,
+                                    (act_t*)out + (size_t)r * N, rows, N, gate, st);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------- RMS norm of a run of columns, written several times
+// out[t][c * Rp + i] = in[t][i] / sqrt(mean_i(in[t][i]^2) + eps) * w[i] for i < R, 0 for R <= i < Rp, for the copies
+// c = 0 .. copies - 1: the normed latent of an attention that keeps one compressed row per position, laid where the
+// cache write expects a key row and a value row (both are that latent), padded to the kernels' width.  A wave a token.
+template <class W>
+__global__ __launch_bounds__(256) void latent_norm_kernel(const float* __restrict__ in, int64_t ld_in, const W* __restrict__ w,
+                                                          float eps, float* __restrict__ out, int64_t ld_out, int copies,
+                                                          int R, int Rp, int T) {
+  const int t = blockIdx.x * 4 + threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  if (t >= T) return;
+  const float* row = in + (size_t)t * ld_in;
+  float ss = 0.f;
+  for (int i = lane; i < R; i += TQ_WAVE) ss += row[i] * row[i];
+  ss = wave_sum(ss);
+  const float rs = 1.0f / sqrtf(ss / (float)R + eps);
+  for (int i = lane; i < Rp; i += TQ_WAVE) {
+    const float v = i < R ? row[i] * rs * to_f32(w[i]) : 0.f;
+    for (int c = 0; c < copies; ++c) out[(size_t)t * ld_out + (size_t)c * Rp + i] = v;
+  }
+}
+
+TQ_API int tq_latent_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, float* out, int64_t ld_out,
+                          int copies, int R, int Rp, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (R < 1 || Rp < R || copies < 1 || ld_in < R || ld_out < (int64_t)copies * Rp || !w) return TQ_ERR_BAD_ARG;
+  TQ_DISPATCH_W(wtype, {
+    hipLaunchKernelGGL(latent_norm_kernel<W>, dim3((T + 3) / 4), dim3(256), 0, st, in, ld_in, (const W*)w, eps, out, ld_out,
+                       copies, R, Rp, T);
+  });
   TQ_LAUNCH_CHECK();
   return 0;
 }
@@ -269,7 +346,8 @@ TQ_API int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, in
 // /root/reference/src/engine/tq_transformer.c:1111-1124, with the formula of tq_ops.c:1373-1410.  A wave per head.
 template <class W>
 __global__ __launch_bounds__(256) void head_rmsnorm_kernel(float* __restrict__ qkv, const W* __restrict__ wq,
-                                                           const W* __restrict__ wk, float eps, int nh, int nkv, int hd) {
+                                                           const W* __restrict__ wk, float eps, int nh, int nkv, int hd,
+                                                           int norm_dim) {
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   const int head = blockIdx.y * 4 + wave;
   if (head >= nh + nkv) return;
@@ -278,18 +356,18 @@ __global__ __launch_bounds__(256) void head_rmsnorm_kernel(float* __restrict__ q
   float* x = qkv + ((size_t)blockIdx.x * (nh + 2 * nkv) + head) * hd;
   float ss = 0.f;
   for (int i = lane; i < hd; i += TQ_WAVE) ss = fmaf(x[i], x[i], ss);
-  ss = wave_sum(ss) / (float)hd + eps;
+  ss = wave_sum(ss) / (float)norm_dim + eps;      // (heads laid out wider than they are hold zeros behind their norm_dim values)
   const float rs = 1.0f / sqrtf(ss);
   for (int i = lane; i < hd; i += TQ_WAVE) x[i] = x[i] * rs * to_f32(w[i]);
 }
 
 TQ_API int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype, float eps, int T, int nh, int nkv,
-                           int hd, hipStream_t st) {
+                           int hd, int norm_dim, hipStream_t st) {
   if (T <= 0 || (!wq && !wk)) return 0;
-  if (nh < 0 || nkv < 0 || hd < 1 || (nh + nkv + 3) / 4 > 65535) return TQ_ERR_BAD_ARG;
+  if (nh < 0 || nkv < 0 || hd < 1 || norm_dim < 1 || norm_dim > hd || (nh + nkv + 3) / 4 > 65535) return TQ_ERR_BAD_ARG;
   TQ_DISPATCH_W(wtype, {
     hipLaunchKernelGGL(head_rmsnorm_kernel<W>, dim3(T, (nh + nkv + 3) / 4), dim3(256), 0, st, qkv, (const W*)wq,
-                       (const W*)wk, eps, nh, nkv, hd);
+                       (const W*)wk, eps, nh, nkv, hd, norm_dim);
   });
   TQ_LAUNCH_CHECK();
   return 0;
@@ -639,6 +717,7 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
       const float a = xr[i + u] + (v[i + u] * rd) * to_f32(wd[i + u]);
       v[i + u] = a;
       if (!rows) xr[i + u] = a;
+      if (!w && out) out[(size_t)r * H + i + u] = from_f32<act_t>(a);      // the summed stream itself, for a part that reads it un-normed
       s2 += a * a;
     }
   }
@@ -656,7 +735,7 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
 }
 
 // As tq_add_rmsnorm, with the weights wd and the eps_d of the norm that what is added passes first; w null: the
-// stream is summed and nothing is normed (no out, no out32).
+// stream is summed and nothing is normed (no out32; `out`, if given, receives the summed stream in the activation type).
 TQ_API int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
                                  const int* pair_slot, const float* weights, int topk, const float* gate,
                                  const void* wd, float eps_d, const void* w, int wtype, float eps, const int* rows,

@@ -34,9 +34,10 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 _SIGNATURES = {
     "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
     "tq_softcap": [_c_ptr, _c_i64, _c_f32, _c_ptr],
+    "tq_scale_softcap": [_c_ptr, _c_i64, _c_f32, _c_f32, _c_ptr],
     "tq_move_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr],
     "tq_gated_act": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "tq_head_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_head_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
                        _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -61,7 +62,19 @@ _SIGNATURES = {
     "tq_add_normed_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr,
                               _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_attention_generic_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
-                                 _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
+                                 _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "tq_act_rows": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_latent_norm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_head_gemm": [_c_ptr, _c_int, _c_i64, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
+                     _c_int, _c_int, _c_ptr],
+    "tq_delta_prep_h": [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                        _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_delta_scan_h": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                        _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_delta_out_h": [_c_ptr, _c_ptr, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_delta_decode_h": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                          _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_router_topk_grouped": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_route_grouped": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
@@ -96,11 +109,11 @@ _OPTIONAL = {
     "tq_probe_mfma": [_c_int, _c_int, _c_int, ctypes.c_uint, _c_ptr, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_f32_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
-                             _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
-                             _c_int, _c_ptr],
+                             _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                             _c_int, _c_int, _c_ptr],
     "tq_attention_mfma_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
-                              _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
-                              _c_int, _c_ptr],
+                              _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                              _c_int, _c_int, _c_ptr],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
@@ -189,7 +202,8 @@ _PROFILE: list | None = None
 _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pair": "matmul", "qkv_rope_write": "matmul",
          "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
          "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
-         "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn"}
+         "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn",
+         "head_gemm": "matmul", "latent_norm": "attn"}
 
 
 def profile_begin() -> None:
@@ -259,10 +273,14 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, act, scale: float = 1.0, po
     return x
 
 
-def softcap(logits: torch.Tensor, cap: float, act) -> torch.Tensor:
-    """logits <- cap * tanh(logits / cap), in place."""
+def softcap(logits: torch.Tensor, cap: float | None, act, scale: float = 1.0) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place; with ``scale``, of the logits times it (``cap`` None: that alone)."""
     k = "softcap"
     _check(logits, k, "logits", torch.float32)
+    if scale != 1.0 or cap is None:
+        _need(cap is None or cap > 0, k, "the cap must be positive")
+        _run(k, library(act).tq_scale_softcap(_ptr(logits), logits.numel(), float(scale), float(cap or 0.0), _stream()))
+        return logits
     _need(cap > 0, k, "the cap must be positive")
     _run(k, library(act).tq_softcap(_ptr(logits), logits.numel(), float(cap), _stream()))
     return logits
@@ -325,23 +343,30 @@ class NormedDelta:
 
 
 def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float, act,
-                rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False):
+                rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False, stream: bool = False):
     """x += delta (in place, unless ``rows`` picks rows), where delta is None, float32 partial sums [S, T, H] added
     one after the other, a GatheredSum, or a NormedDelta around either (then what is added is its RMS norm); returns
     rmsnorm(x) * weight as (activation-typed or None, float32 or None), one row per entry of ``rows`` (all rows if
-    None).  ``weight`` None (with a NormedDelta only): the stream is summed and nothing is returned."""
+    None).  ``weight`` None (with a NormedDelta only): the stream is summed and nothing is returned.  ``stream`` (with
+    ``weight`` None, and delta None or a NormedDelta): the summed stream itself is returned in the activation type, for
+    a part that reads the stream un-normed (on the float32 library that is ``x``, which the next sum changes)."""
     k = "add_rmsnorm"
     _check(x, k, "x", torch.float32)
     _need(x.dim() == 2, k, "x must be [T, H]")
     T, H = x.shape
     post = None
+    if stream:
+        _need(weight is None and rows is None and (delta is None or isinstance(delta, NormedDelta)), k,
+              "the stream itself is returned for all rows, behind nothing or a normed part")
+        if delta is None:
+            return (x if dtype_name(act) == "float32" else act_rows(x, None, None, act)), None
     if isinstance(delta, NormedDelta):
         post, delta = delta, delta.inner
         _check(post.weight, k, "the added part's norm weight", tuple(_WTYPE), (H,))
         _need(delta is not None, k, "a normed part needs something to norm")
     if weight is None:
         _need(post is not None and rows is None, k, "without a weight only a normed part can be summed, into all rows")
-        want_act = want_f32 = False
+        want_act, want_f32 = stream and dtype_name(act) != "float32", False
     else:
         _check(weight, k, "weight", tuple(_WTYPE), (H,))
         _need(post is None or post.weight.dtype == weight.dtype, k, "the two norms' weights must have one type")
@@ -376,7 +401,7 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float,
                                                    topk, _ptr(gate), _ptr(post.weight), float(post.eps), _ptr(weight),
                                                    _WTYPE[post.weight.dtype], float(eps), _ptr(rows), R, _ptr(out),
                                                    _ptr(out32), H, _stream()))
-        return out, out32
+        return (x if stream and out is None else out), out32
     _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights), topk,
                                         _ptr(gate), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(rows), R,
                                         _ptr(out), _ptr(out32), H, _stream()))
@@ -384,9 +409,11 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float,
 
 
 def head_rmsnorm(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
-                 num_heads: int, num_kv_heads: int, head_dim: int, act) -> torch.Tensor:
+                 num_heads: int, num_kv_heads: int, head_dim: int, act, norm_dim: int | None = None) -> torch.Tensor:
     """RMS norm of every query head (weights ``q_weight`` [hd]) and key head (``k_weight``) of the float32 rows
-    ``qkv`` [T, (nh + 2 nkv) * hd], in place; None leaves those heads alone.  Returns ``qkv``."""
+    ``qkv`` [T, (nh + 2 nkv) * hd], in place; None leaves those heads alone.  ``norm_dim``: the values a head really
+    has, where heads are laid out wider (zeros behind them, in the rows and in the weights): the mean is over these.
+    Returns ``qkv``."""
     k = "head_rmsnorm"
     _check(qkv, k, "qkv", torch.float32)
     _need(qkv.dim() == 2 and qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim, k,
@@ -399,7 +426,8 @@ def head_rmsnorm(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: tor
             wtype = w.dtype
     if wtype is not None:
         _run(k, library(act).tq_head_rmsnorm(_ptr(qkv), _ptr(q_weight), _ptr(k_weight), _WTYPE[wtype], float(eps),
-                                             qkv.shape[0], num_heads, num_kv_heads, head_dim, _stream()))
+                                             qkv.shape[0], num_heads, num_kv_heads, head_dim,
+                                             head_dim if norm_dim is None else int(norm_dim), _stream()))
     return qkv
 
 
@@ -842,12 +870,14 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
               positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, page_size: int,
               page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
               scale: float, act, runs: dict | None = None, softcap: float | None = None,
-              distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None) -> torch.Tensor:
+              distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None,
+              sink: torch.Tensor | None = None) -> torch.Tensor:
     """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
 
     ``softcap`` c: a scaled score s becomes c tanh(s / c).  ``distance_bias`` (r1, r2), float32 [nh] each: then
     r1[h] ln(1 + r2[h] (i - j)) is taken off the score of query position i and key position j.  ``chunk`` n: position i
-    sees j only if i // n == j // n, beside j <= i and the window.
+    sees j only if i // n == j // n, beside j <= i and the window.  ``sink`` float32 [nh]: the softmax's denominator of
+    head h also holds exp(sink[h]), a score without key and value that is neither scaled nor capped and counts once.
 
     ``seq_of_token`` gives each token's row of ``block_table`` (its slot).  ``runs`` describes the same tokens
     as runs of consecutive positions, one per sequence, for the kernels that work on tiles of tokens:
@@ -876,7 +906,9 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
         r1, r2 = distance_bias
         _check(r1, k, "r1", torch.float32, (num_heads,))
         _check(r2, k, "r2", torch.float32, (num_heads,))
-    mod = (cap, _ptr(r1), _ptr(r2), int(chunk or 0))
+    if sink is not None:
+        _check(sink, k, "sink", torch.float32, (num_heads,))
+    mod = (cap, _ptr(r1), _ptr(r2), int(chunk or 0), _ptr(sink))
     if (runs is not None and dtype_name(act) == "bfloat16" and hasattr(lib, "tq_attention_mfma")
             and head_dim % 16 == 0 and head_dim <= 256 and page_size % 64 == 0 and page_stride % 8 == 0 and scale > 0):
         B = runs["slots"].numel()
@@ -1020,6 +1052,7 @@ class DeltaDims:
     taps: int
     rank_a: int
     rank_g: int
+    head_decay: bool = False      # one decay per head from a projection of its own, a full gate; no ranks
 
     @property
     def channels(self) -> int:
@@ -1027,6 +1060,8 @@ class DeltaDims:
 
     @property
     def projections(self) -> int:
+        if self.head_decay:        # q | k | v | b (H) | a (H) | gate (H V)
+            return self.channels + 2 * self.heads + self.heads * self.vdim
         return self.channels + self.heads + self.rank_a + self.rank_g
 
     @property
@@ -1156,6 +1191,161 @@ def delta_decode(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: tor
                                          _WTYPE[low_weight.dtype], _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), float(eps),
                                          _ptr(proj), _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride,
                                          *dims.sizes(), dims.rank_a, dims.rank_g, B, _ptr(out), _stream()))
+    return out
+
+
+def _delta_runs(k: str, runs: dict):
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    return B
+
+
+def delta_prep_h(proj: torch.Tensor, slot_of_token: torch.Tensor, state: torch.Tensor, conv_w: torch.Tensor,
+                 a_log: torch.Tensor, dt_bias: torch.Tensor, dims: DeltaDims, act):
+    """The form of ``delta_prep`` with one decay per head: from the float32 projections [T, q | k | v | b | a | gate]
+    q, k, v and beta as there, and dec = exp(-exp(a_log[h]) softplus(a + dt_bias[h])), float32 [T, H]."""
+    k = "delta_prep"
+    T = slot_of_token.numel()
+    _need(dims.head_decay, k, "the sizes must be those of the form with a decay per head")
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    _check(slot_of_token, k, "slot_of_token", torch.int32, (T,))
+    stride = _delta_state(k, state, dims)
+    _check(conv_w, k, "conv_w", torch.float32, (dims.channels, dims.taps))
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    _check(a_log, k, "a_log", torch.float32, (H,))
+    _check(dt_bias, k, "dt_bias", torch.float32, (H,))
+    dev, f32 = proj.device, torch.float32
+    qn = torch.empty((T, G * D), dtype=f32, device=dev)
+    kn = torch.empty((T, G * D), dtype=f32, device=dev)
+    vc = torch.empty((T, H * V), dtype=f32, device=dev)
+    beta = torch.empty((T, H), dtype=f32, device=dev)
+    dec = torch.empty((T, H), dtype=f32, device=dev)
+    _run(k, library(act).tq_delta_prep_h(_ptr(proj), _ptr(slot_of_token), _ptr(state), stride, _ptr(conv_w), _ptr(a_log),
+                                         _ptr(dt_bias), *dims.sizes(), _ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(dec), T,
+                                         _stream()))
+    return qn, kn, vc, beta, dec
+
+
+def delta_scan_h(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, dec: torch.Tensor, runs: dict,
+                 state: torch.Tensor, dims: DeltaDims, act) -> torch.Tensor:
+    """The recurrence of ``delta_scan`` with the whole state of a head decaying by dec[t, h] before token t's write."""
+    k = "delta_scan"
+    T = qn.shape[0]
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    for name, t, w in (("qn", qn, G * D), ("kn", kn, G * D), ("vc", vc, H * V), ("beta", beta, H), ("dec", dec, H)):
+        _check(t, k, name, torch.float32, (T, w))
+    stride = _delta_state(k, state, dims)
+    B = _delta_runs(k, runs)
+    o = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)
+    _run(k, library(act).tq_delta_scan_h(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(dec), _ptr(runs["cu_seqlens"]),
+                                         _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), T, B, _ptr(o), _stream()))
+    return o
+
+
+def delta_out_h(o: torch.Tensor, norm_w: torch.Tensor, eps: float, proj: torch.Tensor, gate: str, runs: dict,
+                state: torch.Tensor, dims: DeltaDims, act) -> torch.Tensor:
+    """As ``delta_out``, the gate being activation ``gate`` (a name of GATES) of the last H*vdim columns of ``proj``."""
+    k = "delta_out"
+    T = o.shape[0]
+    H, V = dims.heads, dims.vdim
+    _check(o, k, "o", torch.float32, (T, H * V))
+    _check(norm_w, k, "norm_w", torch.float32, (V,))
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    stride = _delta_state(k, state, dims)
+    B = _delta_runs(k, runs)
+    out = torch.empty((T, H * V), dtype=ACT_DTYPES[dtype_name(act)], device=o.device)
+    _run(k, library(act).tq_delta_out_h(_ptr(o), _ptr(norm_w), float(eps), _ptr(proj), _gate_code(k, gate),
+                                        _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), T, B,
+                                        _ptr(out), _stream()))
+    return out
+
+
+def delta_decode_h(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, a_log: torch.Tensor,
+                   dt_bias: torch.Tensor, norm_w: torch.Tensor, eps: float, proj: torch.Tensor, gate: str, runs: dict,
+                   state: torch.Tensor, dims: DeltaDims, act) -> torch.Tensor:
+    """A decode step of the form with a decay per head, from ``delta_prep_h``'s outputs to the mixer's output
+    [T, H*vdim] in the activation type, in one launch."""
+    k = "delta_decode"
+    T = qn.shape[0]
+    G, D, H, V = dims.kv_heads, dims.dim, dims.heads, dims.vdim
+    for name, t, w in (("qn", qn, G * D), ("kn", kn, G * D), ("vc", vc, H * V), ("beta", beta, H)):
+        _check(t, k, name, torch.float32, (T, w))
+    _check(a_log, k, "a_log", torch.float32, (H,))
+    _check(dt_bias, k, "dt_bias", torch.float32, (H,))
+    _check(norm_w, k, "norm_w", torch.float32, (V,))
+    _check(proj, k, "proj", torch.float32, (T, dims.projections))
+    stride = _delta_state(k, state, dims)
+    B = _delta_runs(k, runs)
+    _need(T == B and runs["decode"], k, "a decode step brings one token per sequence")
+    _need(delta_decode_fits(dims), k, "a head's lanes do not fit one workgroup")
+    out = torch.empty((T, H * V), dtype=ACT_DTYPES[dtype_name(act)], device=qn.device)
+    _run(k, library(act).tq_delta_decode_h(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(a_log), _ptr(dt_bias), _ptr(norm_w),
+                                           float(eps), _ptr(proj), _gate_code(k, gate), _ptr(runs["cu_seqlens"]),
+                                           _ptr(runs["slots"]), _ptr(state), stride, *dims.sizes(), B, _ptr(out), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ products per head, and what goes with them
+def act_rows(g: torch.Tensor, u: torch.Tensor | None, activation: str | None, act) -> torch.Tensor:
+    """f(g) * u in the activation type, row by row: ``g`` and ``u`` float32 [M, N] whose rows may be runs of columns
+    of wider tensors (unit stride along a row); ``u`` None: f(g) alone; ``activation`` None: no f (with ``u`` None
+    that is a change of type)."""
+    k = "act_rows"
+    for name, t in (("g", g), ("u", u)):
+        if t is not None:
+            _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1,
+                  k, lambda: f"{name} must be float32 [M, N] on the GPU with unit stride along its rows")
+    M, N = g.shape
+    _need(u is None or tuple(u.shape) == (M, N), k, "g and u must have one shape")
+    out = torch.empty((M, N), dtype=ACT_DTYPES[dtype_name(act)], device=g.device)
+    code = -1 if activation is None else _gate_code(k, activation)
+    _run(k, library(act).tq_act_rows(_ptr(g), g.stride(0), _ptr(u), u.stride(0) if u is not None else 0, _ptr(out), M, N,
+                                     code, _stream()))
+    return out
+
+
+def latent_norm(src: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, copies: int, width: int, act) -> None:
+    """RMS norm of the rows of ``src`` (float32 [T, R], a run of columns of a wider tensor allowed) with ``weight`` [R],
+    written ``copies`` times side by side into the rows of ``out`` (float32 [T, copies * width], likewise), each copy
+    padded with zeros to ``width`` columns."""
+    k = "latent_norm"
+    for name, t in (("src", src), ("out", out)):
+        _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1,
+              k, lambda: f"{name} must be float32 [T, n] on the GPU with unit stride along its rows")
+    T, R = src.shape
+    _check(weight, k, "weight", tuple(_WTYPE), (R,))
+    _need(width >= R and copies >= 1 and tuple(out.shape) == (T, copies * width), k,
+          lambda: f"out must be [{T}, {copies * width}], is {tuple(out.shape)}")
+    _run(k, library(act).tq_latent_norm(_ptr(src), src.stride(0), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(out),
+                                        out.stride(0), copies, R, width, T, _stream()))
+
+
+def head_gemm(a: torch.Tensor, w: torch.Tensor, act, out: torch.Tensor | None = None, out_act: bool = False,
+              gate: torch.Tensor | None = None, activation: str = "sigmoid") -> torch.Tensor:
+    """A product per head: out[t, h*N + n] = sum_k a[t, h*K + k] * w[h, n, k], ``w`` [H, N, K].  ``a`` [T, H*K] is
+    float32 or of the activation type, ``out`` [T, H*N] float32 (or the activation type with ``out_act``); both may be
+    runs of columns of wider tensors, and ``out`` may be given.  ``gate`` float32 [T, H*N]: the result is multiplied
+    by ``activation`` (a name of GATES) of it."""
+    k = "head_gemm"
+    adt = ACT_DTYPES[dtype_name(act)]
+    _need(isinstance(w, torch.Tensor) and w.is_cuda and w.dim() == 3 and w.is_contiguous() and w.dtype in _WTYPE, k,
+          "w must be a contiguous [H, N, K] matrix on the GPU")
+    H, N, K = w.shape
+    _need(isinstance(a, torch.Tensor) and a.is_cuda and a.dim() == 2 and a.shape[1] == H * K and a.stride(1) == 1
+          and a.dtype in (torch.float32, adt), k, lambda: f"a must be [T, {H * K}] float32 or {adt} with unit stride along its rows")
+    T = a.shape[0]
+    odt = adt if out_act else torch.float32
+    if out is None:
+        out = torch.empty((T, H * N), dtype=odt, device=a.device)
+    _need(out.is_cuda and out.dtype == odt and tuple(out.shape) == (T, H * N) and out.stride(1) == 1, k,
+          lambda: f"out must be [{T}, {H * N}] {odt} with unit stride along its rows")
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (T, H * N) and gate.stride(1) == 1, k,
+              lambda: f"gate must be float32 [{T}, {H * N}] with unit stride along its rows")
+    _run(k, library(act).tq_head_gemm(_ptr(a), _WTYPE[a.dtype], a.stride(0), _ptr(w), _WTYPE[w.dtype], _ptr(out), int(out_act),
+                                      out.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0,
+                                      _gate_code(k, activation), T, H, N, K, _stream()))
     return out
 
 

@@ -6,6 +6,9 @@
 //                  position i and a key at position j <= i: a bias by distance
 //   chunk > 0      position i sees j only if i / chunk == j / chunk (chunks counted from position 0 of the sequence),
 //                  beside j <= i and beside a window, if there is one
+//   sink           (per query head; null: none) the softmax's denominator also holds exp(sink[h]): a score that has no
+//                  key and no value, is not scaled, capped or biased, and counts once per query.  The kernels start
+//                  their running maximum at sink[h] with a denominator of 1 (the joins of decode steps add it once)
 //
 // All of it in float, on both libraries.
 #pragma once
@@ -16,6 +19,7 @@ struct ScoreMod {
   const float* r1;
   const float* r2;
   int chunk;
+  const float* sink;
 };
 
 // the first position that a token at position p may see

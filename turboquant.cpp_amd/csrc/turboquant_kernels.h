@@ -23,13 +23,17 @@ extern "C" {
 // elementwise.hip: embedding, soft cap, residual sum + RMS norm, per-head norm, rotation + cache write, weighted sum of expert rows (both libraries)
 int tq_embed(const int* tokens, const void* table, int wtype, float* x, int T, int H, float scale, hipStream_t st);
 int tq_softcap(float* x, int64_t n, float cap, hipStream_t st);
+int tq_scale_softcap(float* x, int64_t n, float scale, float cap, hipStream_t st);
 int tq_move_rows(const void* src, const int* idx, void* dst, int n, int64_t row_bytes, int scatter, hipStream_t st);
 int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y, const int* pair_slot,
         const float* weights, int topk, const float* gate, const void* w, int wtype, float eps, const int* rows,
         int R, void* out, float* out32, int H, hipStream_t st);
 int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype, float eps, int T, int nh, int nkv,
-        int hd, hipStream_t st);
+        int hd, int norm_dim, hipStream_t st);
 int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st);
+int tq_act_rows(const float* g, int64_t ldg, const float* u, int64_t ldu, void* out, int M, int N, int gate, hipStream_t st);
+int tq_latent_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, float* out, int64_t ld_out,
+        int copies, int R, int Rp, int T, hipStream_t st);
 int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions,
         const int* seq_of_token, const int* block_table, int bt_stride, const float* inv_freq, int pairing,
         int rot, void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T, int nh, int nkv,
@@ -72,9 +76,9 @@ int tq_attention_generic(const void* q, const void* k_pool, const void* v_pool, 
 int tq_attention_generic_mod(const void* q, const void* k_pool, const void* v_pool, const int* positions,
         const int* seq_of_token, const int* block_table, int bt_stride, int page_size, int64_t page_stride, int T,
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
-        void* out, hipStream_t st);
+        const float* sink, void* out, hipStream_t st);
 // (the *_mod forms of the attention entry points take what score_mod.h describes: a cap on scores, a bias by
-// distance per head, chunks of positions)
+// distance per head, chunks of positions, a sink per head in the softmax's denominator)
 // attention_mfma.hip: bfloat16 attention on the matrix cores (bfloat16 library)
 int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end);
 int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
@@ -84,7 +88,7 @@ int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, con
 int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
-        void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st);
+        const float* sink, void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st);
 // attention_f32.hip: float32 attention on the matrix cores (float32 library)
 int64_t tq_attention_f32_scratch(int B, int nh, int hd, int max_end);
 int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
@@ -94,7 +98,7 @@ int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, cons
 int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
-        void* out, void* partial, int decode, int max_new, int max_end, hipStream_t st);
+        const float* sink, void* out, void* partial, int decode, int max_new, int max_end, hipStream_t st);
 // delta_rule.hip: the gated delta rule over per-sequence state (both libraries)
 int64_t tq_delta_state_floats(int H, int G, int D, int V, int taps);
 int tq_delta_prep(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
@@ -110,6 +114,23 @@ int tq_delta_decode(const float* qn, const float* kn, const float* vc, const flo
         const void* w_low, int wtype, const float* a_log, const float* dt_bias, const float* norm_w, float eps,
         const float* P, const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D,
         int V, int taps, int ra, int rg, int B, void* out, hipStream_t st);
+// (the *_h forms: one decay per head, made from a projection of its own, and a gate with an activation of gates.def)
+int tq_delta_prep_h(const float* P, const int* slot_of_token, const float* state, int64_t state_stride,
+        const float* conv_w, const float* a_log, const float* dt_bias, int H, int G, int D, int V, int taps, float* qn,
+        float* kn, float* vc, float* beta, float* dec, int T, hipStream_t st);
+int tq_delta_scan_h(const float* qn, const float* kn, const float* vc, const float* beta, const float* dec,
+        const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V, int taps,
+        int T, int B, float* o_raw, hipStream_t st);
+int tq_delta_out_h(const float* o_raw, const float* norm_w, float eps, const float* P, int gate_kind,
+        const int* cu_seqlens, const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V, int taps,
+        int T, int B, void* out, hipStream_t st);
+int tq_delta_decode_h(const float* qn, const float* kn, const float* vc, const float* beta, const float* a_log,
+        const float* dt_bias, const float* norm_w, float eps, const float* P, int gate_kind, const int* cu_seqlens,
+        const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V, int taps, int B, void* out,
+        hipStream_t st);
+// head_gemm.hip: a product per head, out[t][h N + n] = sum_k a[t][h K + k] w[h][n][k] (both libraries)
+int tq_head_gemm(const void* a, int a_type, int64_t lda, const void* w, int wtype, void* out, int out_act, int64_t ldc,
+        const float* gate, int64_t ldg, int gate_kind, int T, int H, int N, int K, hipStream_t st);
 // moe.hip: router, choice of experts, order of pairs (both libraries)
 int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
         int* ids, float* weights, float* shared_gate, float* logits, int T, int H, hipStream_t st);

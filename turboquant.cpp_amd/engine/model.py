@@ -138,8 +138,8 @@ class CausalLM:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=x.device)
         normed, _ = self.final_norm.forward(x, pending, ctx, rows=b.want_rows)
         logits = ops.gemm(normed, self.lm_head, self.act)
-        if self.plan.logit_softcap is not None:
-            ops.softcap(logits, self.plan.logit_softcap, self.act)
+        if self.plan.logit_softcap is not None or self.plan.logit_scale != 1.0:
+            ops.softcap(logits, self.plan.logit_softcap, self.act, scale=self.plan.logit_scale)
         return logits
 
 

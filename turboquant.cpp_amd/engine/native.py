@@ -26,6 +26,8 @@ class NativeModel:
         self.lib = host_api.library(model.act)
         if getattr(model, "position_table", None) is not None:
             raise ValueError("the step executor embeds tokens without a learned vector per position")
+        if model.plan.logit_scale != 1.0:
+            raise ValueError("the step executor does not multiply its logits by a constant")
         layers = [b.native() for b in model.blocks]
         if any(l is None for l in layers):
             raise ValueError("a layer of the model has no form in the step executor")

@@ -12,7 +12,9 @@ Options for other designs, all off by default: ``position`` of kind "none" (no r
 ``score_cap`` c (a scaled score s becomes c tanh(s / c)); ``distance_bias`` (two numbers per head, r1 and r2:
 r1 ln(1 + r2 (i - j)) is taken off the score of query position i and key position j); ``chunk`` n (position i sees
 j <= i only if i // n == j // n, chunks counted from position 0 of the sequence); ``value_dim`` (values of another width
-than keys); ``separate_qkv`` (q, k, v and their biases are parameters of their own, joined when the part is prepared).
+than keys); ``separate_qkv`` (q, k, v and their biases are parameters of their own, joined when the part is prepared);
+``sink`` (a learned number per head whose exponential joins the softmax's denominator: a score with no key and no value,
+neither scaled nor capped, counted once).
 With ``separate_qkv`` the heads are laid out at a kernel width that is the larger of key and value width rounded up to
 16: the added rows and columns of the matrices are zeros, which change no score and no output, and every head size
 then runs on the matrix-core kernels of both libraries.
@@ -35,7 +37,7 @@ class GroupedQueryAttention(Part):
                  qkv_bias: bool = False, out_bias: bool = False, window: int | None = None,
                  scale: float | None = None, qk_norm_eps: float | None = None, score_cap: float | None = None,
                  distance_bias: bool = False, chunk: int | None = None, value_dim: int | None = None,
-                 separate_qkv: bool = False):
+                 separate_qkv: bool = False, sink: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         if window is not None and window < 1:
@@ -53,6 +55,7 @@ class GroupedQueryAttention(Part):
         if separate_qkv:
             self.head_dim = -(-max(self.key_dim, self.value_dim) // 16) * 16
         self.r1 = self.r2 = None
+        self.has_sink, self.sink = sink, None
         self.q_weight = self.k_weight = self.v_weight = self.q_bias = self.k_bias = self.v_bias = None
         self.has_qkv_bias, self.has_out_bias, self.window = qkv_bias, out_bias, window
         self.qk_norm_eps = qk_norm_eps
@@ -81,6 +84,10 @@ class GroupedQueryAttention(Part):
                 specs["out_bias"] = ParamSpec((W,), role="bias")
             if self.has_distance_bias:
                 specs.update({"r1": ParamSpec((H,), role="scale"), "r2": ParamSpec((H,), role="scale")})
+            if self.qk_norm_eps is not None:
+                specs.update({"q_norm": ParamSpec((K,), role="scale"), "k_norm": ParamSpec((K,), role="scale")})
+            if self.has_sink:
+                specs["sink"] = ParamSpec((H,), role="scale")
             return specs
         rows = self.q_size + 2 * self.kv_size
         splits = (self.q_size, self.kv_size, self.kv_size)
@@ -97,11 +104,15 @@ class GroupedQueryAttention(Part):
             specs["k_norm"] = ParamSpec((self.head_dim,), role="scale")
         if self.has_distance_bias:
             specs.update({"r1": ParamSpec((self.num_heads,), role="scale"), "r2": ParamSpec((self.num_heads,), role="scale")})
+        if self.has_sink:
+            specs["sink"] = ParamSpec((self.num_heads,), role="scale")
         return specs
 
     def prepare(self, device, act):
         if self.has_distance_bias:      # they enter float arithmetic only
             self.r1, self.r2 = self.r1.float().contiguous(), self.r2.float().contiguous()
+        if self.has_sink:
+            self.sink = self.sink.float().contiguous()
         if not self.separate_qkv or self.qkv_weight is not None:
             return
         D = self.head_dim
@@ -113,6 +124,8 @@ class GroupedQueryAttention(Part):
             return out.view(heads * D, *t.shape[1:])
 
         H, G, K, V = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        if self.qk_norm_eps is not None and K != D:     # zeros behind the head's own values: they norm zeros to zeros
+            self.q_norm, self.k_norm = (torch.cat([w, w.new_zeros(D - K)]) for w in (self.q_norm, self.k_norm))
         self.qkv_weight = torch.cat([heads_padded(self.q_weight, H, K), heads_padded(self.k_weight, G, K),
                                      heads_padded(self.v_weight, G, V)])
         if self.has_qkv_bias:
@@ -137,7 +150,7 @@ class GroupedQueryAttention(Part):
         from ..csrc import host_api
         if self.qk_norm_eps is not None:        # the executor has no form with a norm of the heads
             return None
-        if self.score_cap is not None or self.has_distance_bias or self.chunk is not None or self.separate_qkv:
+        if self.score_cap is not None or self.has_distance_bias or self.chunk is not None or self.separate_qkv or self.has_sink:
             return None                         # nor one with changed scores or chunks
         table = self.position.table(self.qkv_weight.device)
         if table.dtype != torch.float32 or not table.is_contiguous() or table.numel() * 2 != self.position.rotary_dim:
@@ -156,6 +169,8 @@ class GroupedQueryAttention(Part):
             opts["distance_bias"] = (self.r1, self.r2)
         if self.chunk is not None:
             opts["chunk"] = self.chunk
+        if self.has_sink:
+            opts["sink"] = self.sink
         return opts
 
     def forward(self, normed, ctx, entry):
@@ -168,7 +183,7 @@ class GroupedQueryAttention(Part):
         else:
             qkv = ops.gemm(normed, self.qkv_weight, ctx.act, bias=self.qkv_bias)
             ops.head_rmsnorm(qkv, self.q_norm, self.k_norm, self.qk_norm_eps, self.num_heads, self.num_kv_heads,
-                             self.head_dim, ctx.act)
+                             self.head_dim, ctx.act, norm_dim=self.key_dim)
             q = ops.rope_kv_write(qkv, *rope, runs=b.runs())
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,

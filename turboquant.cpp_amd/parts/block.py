@@ -87,3 +87,41 @@ class SandwichBlock(Part):
         want32 = getattr(self.ffn, "wants_f32", False)
         normed, normed32 = self.ffn_norm.forward(x, pending, ctx, want_f32=want32)
         return ops.NormedDelta(self.ffn.forward(normed, normed32, ctx), self.ffn_post_norm.weight, self.ffn_post_norm.eps)
+
+
+@register_part("block", "outnorm")
+class OutputNormBlock(Part):
+    """A norm on every part's output only: ``x += norm_a(mixer(x)); x += norm_b(ffn(x))``.  The parts read the residual
+    stream itself, un-normed, in the activation type; the feed-forward half is optional (``ffn`` and ``ffn_norm`` None: the
+    layer is its mixer alone).  A part's output travels on wrapped with the weights of its norm (``ops.NormedDelta``), and
+    the kernel that sums it into the stream norms it in the same pass and hands the summed stream to the next part."""
+    graph_safe = True
+    slots = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "ffn", "ffn_norm": "norm"}
+    optional = ("ffn", "ffn_norm")
+
+    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a layer has a feed-forward with its norm, or neither")
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+
+    def children(self):
+        parts = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "ffn": self.ffn, "ffn_norm": self.ffn_norm}
+        return {k: v for k, v in parts.items() if v is not None}
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def forward(self, x, pending, ctx, entry):
+        from ..csrc import ops
+        if pending is not None and not isinstance(pending, ops.NormedDelta):     # a layer of another arrangement before this one
+            ops.add_rmsnorm(x, pending, self.mixer_norm.weight, self.mixer_norm.eps, ctx.act, want_act=False)
+            pending = None
+        h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
+        pending = ops.NormedDelta(self.mixer.forward(h, ctx, entry), self.mixer_norm.weight, self.mixer_norm.eps)
+        if self.ffn is None:
+            return pending
+        h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
+        return ops.NormedDelta(self.ffn.forward(h, None, ctx), self.ffn_norm.weight, self.ffn_norm.eps)

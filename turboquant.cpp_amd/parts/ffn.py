@@ -1,4 +1,5 @@
-"""Feed-forward parts: a dense gated one and a sparse one with routed experts and a shared expert.
+"""Feed-forward parts: a dense gated one, a dense one with an activation and no gate, and a sparse one with routed
+experts and a shared expert.
 
 Dense (/root/reference/src/engine/tq_transformer.c:2707-2824): ``down(silu(gate x) * (up x))``, no biases; the
 gate's activation is an argument (``silu``, ``gelu_tanh`` as /root/reference/src/engine/tq_ops.c:1482-1484, ``relu2``)
@@ -53,6 +54,28 @@ class DenseSwiGLU(Part):
 
     def forward(self, normed, normed32, ctx):
         h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True, activation=self.activation)
+        return ops.gemm(h, self.down, ctx.act, partial_sums=True)
+
+
+@register_part("ffn", "dense_act")
+class DenseActivated(Part):
+    """Two matrices and an activation between them, no gate and no biases: ``down(f(up x))``, f one of the activations
+    of ``ops.GATES`` (``relu2``: the square of relu)."""
+    graph_safe = True
+    wants_f32 = False
+
+    def __init__(self, hidden_size: int, inner_size: int, activation: str = "relu2"):
+        if activation not in ops.GATES:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(sorted(ops.GATES))}")
+        self.hidden_size, self.inner_size, self.activation = hidden_size, inner_size, activation
+        self.up = self.down = None
+
+    def param_specs(self):
+        return {"up": ParamSpec((self.inner_size, self.hidden_size)),
+                "down": ParamSpec((self.hidden_size, self.inner_size))}
+
+    def forward(self, normed, normed32, ctx):
+        h = ops.act_rows(ops.gemm(normed, self.up, ctx.act), None, self.activation, ctx.act)
         return ops.gemm(h, self.down, ctx.act, partial_sums=True)
 
 
