@@ -15,6 +15,12 @@ time the other two workloads: a batch of prompts of unequal lengths in one promp
 times the Felepel design (delta-rule and chunked-attention layers, experts chosen within groups) beside Qwen2-MoE at
 equal sizes: prompt steps of 512 and 2,048 tokens, decode steps at batch 1 and 8, and where each model's time goes,
 kernel by kernel.  The default run and its line are not touched by it.
+
+    python bench.py --design taminex [--design-sizes small,medium] [--layers 8]
+
+does the same for the Taminex design (a norm on every part's output only; attention with head norms, partial rotation
+and a sink; the delta rule with a decay per head; attention over a latent per position, shared between layers; a
+feed-forward of two matrices with squared relu) beside Qwen2-MoE with dense feed-forwards of as many weights.
 """
 from __future__ import annotations
 
@@ -239,11 +245,15 @@ def unequal_workload(sizes: str, act: str, layers: int | None, wl: dict) -> dict
 
 
 # ---------------------------------------------------------------- the Felepel design beside Qwen2-MoE at equal sizes
-# name -> width, heads, kv heads of the attention, head size, experts, groups, kept groups, experts per token, expert width
+# name -> width, heads, kv heads of the attention, head size, experts, groups, kept groups, experts per token, expert width;
+# for Taminex the width of a dense gated feed-forward and the latent's size
 DESIGN_SIZES = {
-    "small": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=32, groups=4, keep=2, top=4, ff=768, vocab=32000),
-    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=64, groups=8, keep=2, top=4, ff=1408, vocab=32000),
-    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=32, groups=4, keep=1, top=2, ff=4096, vocab=32000),
+    "small": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=32, groups=4, keep=2, top=4, ff=768, vocab=32000,
+                  dense_ff=2816, kv_rank=256),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=64, groups=8, keep=2, top=4, ff=1408, vocab=32000,
+                   dense_ff=5632, kv_rank=512),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=32, groups=4, keep=1, top=2, ff=4096, vocab=32000,
+                  dense_ff=11008, kv_rank=512),
 }
 
 
@@ -265,6 +275,35 @@ def felepel_config(z: dict, layers: int, max_positions: int) -> dict:
             "norm": {"eps": 1e-5}, "layers": out}
 
 
+def taminex_config(z: dict, layers: int, max_positions: int) -> dict:
+    """`layers` layers in the order delta rule, attention, latent attention, latent attention on the layer before's
+    latents; a feed-forward of two matrices, half as wide again as the gated one of three beside it."""
+    mlp = {"kind": "dense", "ff": z["dense_ff"] * 3 // 2}
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    kinds = [
+        {"type": "delta", "mixer": {"heads": H, "kv_heads": H, "dim": D, "vdim": D, "conv": 4}},
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                                        "rot": {"dims": D // 2, "base": 1e6}}},
+        {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": z["kv_rank"], "scale": D ** -0.5}},
+        {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": z["kv_rank"], "scale": D ** -0.5}},
+    ]
+    out = []
+    for i in range(layers):
+        layer = {"type": kinds[i % 4]["type"], "mixer": dict(kinds[i % 4]["mixer"]), "mlp": mlp}
+        if i % 4 == 3:
+            layer["mixer"]["kv_from"] = i - 1
+        out.append(layer)
+    return {"architecture": "Taminex", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+            "logit_softcap": 30.0, "layers": out}
+
+
+def qwen_dense_config_like(z: dict, layers: int, max_positions: int) -> dict:
+    """Qwen2-MoE's layers with the dense gated feed-forward in every layer (`mlp_only_layers`)."""
+    return dict(A27B, vocab_size=z["vocab"], hidden_size=z["width"], num_hidden_layers=layers, num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=z["dense_ff"],
+                mlp_only_layers=list(range(layers)), max_window_layers=layers, max_position_embeddings=max_positions)
+
+
 def qwen_config_like(z: dict, layers: int, max_positions: int) -> dict:
     return dict(A27B, vocab_size=z["vocab"], hidden_size=z["width"], num_hidden_layers=layers, num_attention_heads=z["heads"],
                 num_key_value_heads=z["kv_heads"], head_dim=z["dim"], moe_intermediate_size=z["ff"],
@@ -279,9 +318,11 @@ def design_comparison(args) -> int:
     from turboquant_cpp_amd.engine.step import Engine
     act, dev = args.dtype, "cuda:0"
     short = "bf16" if act == "bfloat16" else "fp32"
-    layers = args.layers or 6
+    layers = args.layers or (8 if args.design == "taminex" else 6)
     context, prompts_at, batches = 2048, (512, 2048), (1, 8)
-    out = {"metric": "Felepel beside Qwen2-MoE at equal sizes: prompt and decode tok/s, and milliseconds by kernel",
+    design = {"felepel": ("Felepel", felepel_config, qwen_config_like),
+              "taminex": ("Taminex", taminex_config, qwen_dense_config_like)}[args.design]
+    out = {"metric": f"{design[0]} beside Qwen2-MoE at equal sizes: prompt and decode tok/s, and milliseconds by kernel",
            "unit": "tok/s", "dtype": short, "layer_runs": layers, "data": "synthetic", "sizes": {}}
 
     def measure(cfg):
@@ -344,8 +385,8 @@ def design_comparison(args) -> int:
     for name in args.design_sizes.split(","):
         z = DESIGN_SIZES[name]
         out["sizes"][name] = {"config": z,
-                              "felepel": measure(felepel_config(z, layers, context + 64)),
-                              "qwen2_moe": measure(qwen_config_like(z, layers, context + 64))}
+                              args.design: measure(design[1](z, layers, context + 64)),
+                              "qwen2_moe": measure(design[2](z, layers, context + 64))}
         print(f"[bench] {name} done", file=sys.stderr, flush=True)
     print(json.dumps(out), flush=True)
     return 0
@@ -384,7 +425,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--no-workloads", action="store_true",
                     help="leave out the two workloads of unequal prompts that the default run adds under \"workloads\"")
-    ap.add_argument("--design", default=None, choices=["felepel"],
+    ap.add_argument("--design", default=None, choices=["felepel", "taminex"],
                     help="time this design beside Qwen2-MoE at equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="of " + ", ".join(DESIGN_SIZES))
     args = ap.parse_args()
