@@ -76,6 +76,12 @@ CASES = {
         (delta(2, 1, 192, 272, conv=3), None),
         (latent(2, 32, 48, 304), None),
     ], logit_scale=2.5, logit_softcap=40.0),
+    # latents as wide as the attention kernels take them, and just below
+    "widest": config(128, 200, [
+        (latent(2, 32, 32, 512), dense(64)),
+        (latent(4, 16, 16, 512, kv_from=0), None),
+        (latent(2, 32, 16, 496), None),
+    ], logit_softcap=20.0),
     # as a served model's layers might be laid out, small
     "regular": config(128, 256, [
         (delta(4, 2, 32, 32), dense(256)),

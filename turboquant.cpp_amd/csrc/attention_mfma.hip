@@ -242,19 +242,23 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     for (int g = 0; g < QG; ++g) s[g][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (ONCE) {
       const int row_a = 32 * (jt / 2) + 8 * (r8 / 4) + 4 * (jt % 2) + r8 % 4, row_b = row_a + 16;
-      u32x4 kf[KS];
+      constexpr int KG = KS > 8 ? 8 : KS;      // steps of hd whose keys a lane holds at a time (heads beyond 256: half of them)
 #pragma unroll
-      for (int p = 0; p < KS / 2; ++p) {
-        kf[2 * p] = ld16_once(kt + row_a * k_stride + 64 * p + q8);
-        kf[2 * p + 1] = ld16_once(kt + row_b * k_stride + 64 * p + q8);
+      for (int k0 = 0; k0 < KS; k0 += KG) {
+        u32x4 kf[KG];
+#pragma unroll
+        for (int p = 0; p < KG / 2; ++p) {
+          kf[2 * p] = ld16_once(kt + row_a * k_stride + 64 * (k0 / 2 + p) + q8);
+          kf[2 * p + 1] = ld16_once(kt + row_b * k_stride + 64 * (k0 / 2 + p) + q8);
+        }
+#pragma unroll
+        for (int p = 0; p < KG / 2; ++p) to_own_row(kf[2 * p], kf[2 * p + 1]);
+#pragma unroll
+        for (int ks = 0; ks < KG; ++ks)
+#pragma unroll
+          for (int g = 0; g < QG; ++g)
+            s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[ks]), qf[g][k0 + ks], s[g][jt], 0, 0, 0);
       }
-#pragma unroll
-      for (int p = 0; p < KS / 2; ++p) to_own_row(kf[2 * p], kf[2 * p + 1]);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int g = 0; g < QG; ++g)
-          s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[ks]), qf[g][ks], s[g][jt], 0, 0, 0);
       continue;
     }
 #pragma unroll
@@ -422,8 +426,12 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 #define KPAD 8
 #define VSTR 72
 
+// Heads wider than 256 (DT = 32; an attention over compressed rows that all heads share has such): one buffer instead of
+// two, since two tiles of 64 x 512 keys and values are beyond the LDS, and a wave to a SIMD, since a column's sums
+// alone are 128 registers; the next tile still travels from memory into registers while this one is worked on.
 template <int DT, int QG, bool EXACT, bool MOD>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1 : 2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
+  constexpr bool ONEBUF = DT > 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int QW = 16 * QG;
   constexpr int KCH = (TILE * 2 * DT + 255) / 256;      // 16-byte chunks of a key tile per thread
@@ -482,19 +490,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   // what this thread carries of every tile: where its chunks lie in the tile in memory and in LDS (a thread
   // past the end of a small tile carries the last chunk once more)
-  int k_g[KCH], k_l[KCH], v_g[VCH], v_l[VCH];
-#pragma unroll
-  for (int j = 0; j < KCH; ++j) {
+  // (with one buffer the places are worked out anew at every use: 4 (KCH + VCH) registers are more than a wave can spare there)
+  constexpr int NIDX = ONEBUF ? 1 : (KCH > VCH ? KCH : VCH);
+  int k_g_[NIDX], k_l_[NIDX], v_g_[NIDX], v_l_[NIDX];
+  auto k_place = [&](int j, int& in_mem, int& in_lds) {
     const int i = min(tid + j * 256, TILE * kcpr - 1), row = i / kcpr, ch = i % kcpr;
-    k_g[j] = row * hd + ch * 8;
-    k_l[j] = EXACT ? k_swz<DT>(row, ch) : row * kstr + ch * 8;
-  }
-#pragma unroll
-  for (int j = 0; j < VCH; ++j) {
+    in_mem = row * hd + ch * 8;
+    in_lds = EXACT ? k_swz<DT>(row, ch) : row * kstr + ch * 8;
+  };
+  auto v_place = [&](int j, int& in_mem, int& in_lds) {
     const int i = min(tid + j * 256, hd * 8 - 1), d = i / 8, ch = i % 8;
-    v_g[j] = d * a.page_size + ch * 8;
-    v_l[j] = EXACT ? v_swz(d, ch) : d * vstr + ch * 8;
+    in_mem = d * a.page_size + ch * 8;
+    in_lds = EXACT ? v_swz(d, ch) : d * vstr + ch * 8;
+  };
+  if constexpr (!ONEBUF) {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) k_place(j, k_g_[j], k_l_[j]);
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) v_place(j, v_g_[j], v_l_[j]);
   }
+  auto k_g = [&](int j) { if constexpr (ONEBUF) { int m, l; k_place(j, m, l); return m; } else return k_g_[j]; };
+  auto k_l = [&](int j) { if constexpr (ONEBUF) { int m, l; k_place(j, m, l); return l; } else return k_l_[j]; };
+  auto v_g = [&](int j) { if constexpr (ONEBUF) { int m, l; v_place(j, m, l); return m; } else return v_g_[j]; };
+  auto v_l = [&](int j) { if constexpr (ONEBUF) { int m, l; v_place(j, m, l); return l; } else return v_l_[j]; };
   u32x4 pk[KCH], pv[VCH];
   const int tiles_per_page = a.page_size / TILE;
   int page_next = table[tile_beg / tiles_per_page];     // page of the tile that the next fetch takes
@@ -504,17 +522,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int in_page = ((tile) % tiles_per_page) * TILE;                                                   \
     const bf16_t* kg = a.k_pool + base + (int64_t)in_page * hd;                                             \
     const bf16_t* vg = a.v_pool + base + in_page;                                                           \
-    _Pragma("unroll") for (int j = 0; j < KCH; ++j) pk[j] = *reinterpret_cast<const u32x4*>(kg + k_g[j]);   \
-    _Pragma("unroll") for (int j = 0; j < VCH; ++j) pv[j] = *reinterpret_cast<const u32x4*>(vg + v_g[j]);   \
+    _Pragma("unroll") for (int j = 0; j < KCH; ++j) pk[j] = *reinterpret_cast<const u32x4*>(kg + k_g(j));   \
+    _Pragma("unroll") for (int j = 0; j < VCH; ++j) pv[j] = *reinterpret_cast<const u32x4*>(vg + v_g(j));   \
     if ((tile) + 1 < tile_end) page_next = table[((tile) + 1) / tiles_per_page];                            \
   } while (0)
 #define TQ_STAGE(off)                                                                                       \
   do {                                                                                                      \
-    _Pragma("unroll") for (int j = 0; j < KCH; ++j) *reinterpret_cast<u32x4*>(Ks + (off) + k_l[j]) = pk[j]; \
-    _Pragma("unroll") for (int j = 0; j < VCH; ++j) *reinterpret_cast<u32x4*>(Vs + (off) + v_l[j]) = pv[j]; \
+    _Pragma("unroll") for (int j = 0; j < KCH; ++j) *reinterpret_cast<u32x4*>(Ks + (off) + k_l(j)) = pk[j]; \
+    _Pragma("unroll") for (int j = 0; j < VCH; ++j) *reinterpret_cast<u32x4*>(Vs + (off) + v_l(j)) = pv[j]; \
   } while (0)
 
   TQ_FETCH(tile_beg);
+  if constexpr (ONEBUF) {
+    for (int tile = tile_beg; tile < tile_end; ++tile) {
+      TQ_STAGE(0);
+      if (tile + 1 < tile_end) TQ_FETCH(tile + 1);
+      __syncthreads();
+      if (tile >= wave_beg && tile < wave_end) {
+        const int pos0 = tile * TILE;
+        const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
+        tile_step<DT, QG, EXACT, EXACT, false, MOD>(o, m_run, l_run, qf, Ks, kstr, Vs, vstr, hd, pos0, p_q, lo_q,
+                                        a.scale * LOG2E, masked, cm);
+      }
+      __syncthreads();
+    }
+  } else {
   TQ_STAGE(0);
   if (tile_beg + 1 < tile_end) TQ_FETCH(tile_beg + 1);
   __syncthreads();
@@ -531,6 +563,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
                                       a.scale * LOG2E, masked, cm);
     }
     __syncthreads();
+  }
   }
 #undef TQ_FETCH
 #undef TQ_STAGE
@@ -561,7 +594,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // one sequence beyond position 4096 and seven shorter ones a third slower).
 // AHEAD (with EXACT): the form for steps of few waves, which fetches a tile ahead (attend_ahead).
 template <int DT, bool EXACT, bool AHEAD = false, bool MOD = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD || DT > 16 ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.z;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
   const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
@@ -666,7 +699,7 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------ launch
 template <int DT, int QG, bool EXACT, bool MOD>
 static int launch_prefill_as(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  const size_t shmem = 2 * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+  const size_t shmem = (DT > 16 ? 1 : 2) * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT, MOD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
@@ -713,7 +746,7 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
                                  void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st) {
   if (B <= 0) return 0;
   if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
-  if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
+  if (hd % 16 != 0 || hd < 16 || hd > 512 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
   if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
@@ -730,7 +763,9 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
     else if (dt == 16) launch_decode<16, true>(a, B, grid_runs, st);
     else if (dt < 4) launch_decode<4, false>(a, B, grid_runs, st);
     else if (dt < 8) launch_decode<8, false>(a, B, grid_runs, st);
-    else launch_decode<16, false>(a, B, grid_runs, st);
+    else if (dt < 16) launch_decode<16, false>(a, B, grid_runs, st);
+    else if (dt == 32) launch_decode<32, true>(a, B, grid_runs, st);
+    else launch_decode<32, false>(a, B, grid_runs, st);
   } else {
     // two groups of 16 tokens per wave, which halves the reads from LDS per product, when that still leaves
     // the chip two workgroups per compute unit and registers allow; else one group
@@ -741,7 +776,9 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
     else if (dt == 16) rc = launch_prefill<16, 1, true>(a, B, max_new, st);
     else if (dt < 4) rc = two ? launch_prefill<4, 2, false>(a, B, max_new, st) : launch_prefill<4, 1, false>(a, B, max_new, st);
     else if (dt < 8) rc = two ? launch_prefill<8, 2, false>(a, B, max_new, st) : launch_prefill<8, 1, false>(a, B, max_new, st);
-    else rc = launch_prefill<16, 1, false>(a, B, max_new, st);
+    else if (dt < 16) rc = launch_prefill<16, 1, false>(a, B, max_new, st);
+    else if (dt == 32) rc = launch_prefill<32, 1, true>(a, B, max_new, st);
+    else rc = launch_prefill<32, 1, false>(a, B, max_new, st);
     if (rc) return rc;
   }
   TQ_LAUNCH_CHECK();
