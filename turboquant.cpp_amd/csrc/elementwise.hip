@@ -306,6 +306,27 @@ TQ_API int tq_act_rows(const float* g, int64_t ldg, const float* u, int64_t ldu,
   return 0;
 }
 
+// out[m][n] = f(gate[m][n]) * o[m][n]: an output gate on rows that are already in the activation type (an attention's
+// heads), the gate float with a row stride of its own.  In place if out == o.
+__global__ __launch_bounds__(256) void gate_rows_kernel(const act_t* __restrict__ o, const float* __restrict__ gate, int64_t ldg,
+                                                        act_t* __restrict__ out, int N, int kind) {
+  const int m = blockIdx.y;
+  for (int n = blockIdx.x * 256 + threadIdx.x; n < N; n += gridDim.x * 256)
+    out[(size_t)m * N + n] = from_f32<act_t>(to_f32(o[(size_t)m * N + n]) * gate_fn(gate[(size_t)m * ldg + n], kind));
+}
+
+TQ_API int tq_gate_rows(const void* o, const float* gate, int64_t ldg, void* out, int M, int N, int kind, hipStream_t st) {
+  if (M <= 0 || N <= 0) return 0;
+  if (kind < 0 || kind >= TQ_GATE_COUNT || ldg < N) return TQ_ERR_BAD_ARG;
+  for (int r = 0; r < M; r += 65535) {
+    const int rows = M - r < 65535 ? M - r : 65535;
+    hipLaunchKernelGGL(gate_rows_kernel, dim3((N + 1023) / 1024 < 1 ? 1 : (N + 1023) / 1024, rows), dim3(256), 0, st,
+                       (const act_t*)o + (size_t)r * N, gate + (size_t)r * ldg, ldg, (act_t*)out + (size_t)r * N, N, kind);
+  }
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- RMS norm of a run of columns, written several times
 // out[t][c * Rp + i] = in[t][i] / sqrt(mean_i(in[t][i]^2) + eps) * w[i] for i < R, 0 for R <= i < Rp, for the copies
 // c = 0 .. copies - 1: the normed latent of an attention that keeps one compressed row per position, laid where the

@@ -64,6 +64,7 @@ _SIGNATURES = {
     "tq_attention_generic_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
                                  _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "tq_act_rows": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_gate_rows": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_latent_norm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_head_gemm": [_c_ptr, _c_int, _c_i64, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
                      _c_int, _c_int, _c_ptr],
@@ -1303,6 +1304,18 @@ def act_rows(g: torch.Tensor, u: torch.Tensor | None, activation: str | None, ac
     _run(k, library(act).tq_act_rows(_ptr(g), g.stride(0), _ptr(u), u.stride(0) if u is not None else 0, _ptr(out), M, N,
                                      code, _stream()))
     return out
+
+
+def gate_rows(o: torch.Tensor, gate: torch.Tensor, activation: str, act) -> torch.Tensor:
+    """o * f(gate), in place: ``o`` [M, N] contiguous in the activation type, ``gate`` float32 [M, N] whose rows may be
+    runs of columns of a wider tensor, f an activation of GATES."""
+    k = "gate_rows"
+    _check(o, k, "o", ACT_DTYPES[dtype_name(act)])
+    M, N = o.shape
+    _need(isinstance(gate, torch.Tensor) and gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (M, N)
+          and gate.stride(1) == 1, k, lambda: f"gate must be float32 [{M}, {N}] on the GPU with unit stride along its rows")
+    _run(k, library(act).tq_gate_rows(_ptr(o), _ptr(gate), gate.stride(0), _ptr(o), M, N, _gate_code(k, activation), _stream()))
+    return o
 
 
 def latent_norm(src: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, copies: int, width: int, act) -> None:

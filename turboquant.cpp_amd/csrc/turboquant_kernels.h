@@ -32,6 +32,7 @@ int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype, float
         int hd, int norm_dim, hipStream_t st);
 int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st);
 int tq_act_rows(const float* g, int64_t ldg, const float* u, int64_t ldu, void* out, int M, int N, int gate, hipStream_t st);
+int tq_gate_rows(const void* o, const float* gate, int64_t ldg, void* out, int M, int N, int kind, hipStream_t st);
 int tq_latent_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, float* out, int64_t ld_out,
         int copies, int R, int Rp, int T, hipStream_t st);
 int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions,

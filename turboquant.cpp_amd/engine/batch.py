@@ -7,7 +7,7 @@ sequence; a sequence contributes its whole prompt or one decoded token.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import numpy as np
 import torch
@@ -28,6 +28,7 @@ class StepBatch:
     want_rows: torch.Tensor           # int32 [R]: packed rows whose logits are wanted
     n_want: int
     fixed_max_end: int | None = None  # set when launches must not depend on the sequences' true lengths
+    scratch: dict = field(default_factory=dict)      # what parts keep for the rest of the step (see own_pages, shared)
 
     @property
     def n_seqs(self) -> int:
@@ -46,6 +47,27 @@ class StepBatch:
         if self.fixed_max_end is not None:
             return self.fixed_max_end
         return max(s + n for s, n in zip(self.start, self.n_new))
+
+    @property
+    def is_fresh(self) -> bool:
+        """Every sequence of the step starts at its first token: what the step brings is all there is to see."""
+        return all(s == 0 for s in self.start)
+
+    def own_pages(self, page_size: int) -> tuple[torch.Tensor, int]:
+        """A page table for memory that lives for this step only, [highest slot + 1, pages]: the step's sequences get
+        pages of their own for the positions of their new tokens, numbered one after the other; and how many there are.
+        A part that lays out keys and values of its own for the step's tokens finds them through it with the step's
+        slots, as it finds the cache through the cache's table."""
+        key = ("own_pages", page_size)
+        if key not in self.scratch:
+            per = [-(-n // page_size) for n in self.n_new]
+            table = np.zeros((max(self.slots) + 1, max(per)), dtype=np.int32)
+            at = 0
+            for slot, n in zip(self.slots, per):
+                table[slot, :n] = np.arange(at, at + n, dtype=np.int32)
+                at += n
+            self.scratch[key] = (torch.from_numpy(table).to(self.tokens.device), at)
+        return self.scratch[key]
 
     def runs(self) -> dict:
         """The step as runs of consecutive positions, one per sequence, for kernels that tile over tokens."""
