@@ -224,11 +224,14 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][D
 // bytes, eight lanes to a row, and lanes l and l ^ 8 exchange what belongs to the other's row.
 // scale2 = scale * log2(e) > 0: maxima are kept in that unit and probabilities are 2^(s * scale2 - m), which is
 // exp(s * scale - max) with one instruction for the power.
-template <int DT, int QG, bool EXACT, bool SWZ = false, bool ONCE = false, bool MOD = false>
-__device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
+// VD, dt0: the wave sums the VD blocks of 16 value dimensions from block dt0 on (all DT of them unless a step's waves
+// share a head's value dimensions among them); the scores are over all of hd either way.
+template <int DT, int QG, bool EXACT, bool SWZ = false, bool ONCE = false, bool MOD = false, int VD = DT>
+__device__ __forceinline__ void tile_step(f32x4 (&o)[QG][VD], float (&m_run)[QG], float (&l_run)[QG],
                                           const bf16x8 (&qf)[QG][(DT + 1) / 2], const bf16_t* kt, int k_stride,
                                           const bf16_t* vt, int v_stride, int hd, int pos0, const int (&p_q)[QG],
-                                          const int (&lo_q)[QG], float scale2, bool masked, const ColMod<QG, MOD>& cm) {
+                                          const int (&lo_q)[QG], float scale2, bool masked, const ColMod<QG, MOD>& cm,
+                                          int dt0 = 0) {
   constexpr int KS = (DT + 1) / 2;
   const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
   // EXACT: hd == 16 DT with DT even, so nothing below depends on hd and every product is unconditional
@@ -274,12 +277,12 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     }
   }
   bf16x8 pf[2][QG];
-  softmax_tile<DT, QG, MOD>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf, cm);
+  softmax_tile<VD, QG, MOD>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf, cm);
   if (ONCE) {
     // a row of values (64 positions of one dimension) is one line: both halves of the tile come with it
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      u32x4 v0 = ld16_once(vt + (16 * dt + r8) * v_stride + q8), v1 = ld16_once(vt + (16 * dt + 8 + r8) * v_stride + q8);
+    for (int dt = 0; dt < VD; ++dt) {
+      u32x4 v0 = ld16_once(vt + (16 * (dt0 + dt) + r8) * v_stride + q8), v1 = ld16_once(vt + (16 * (dt0 + dt) + 8 + r8) * v_stride + q8);
       to_own_row(v0, v1);
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
@@ -292,9 +295,10 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 #pragma unroll
   for (int pr = 0; pr < 2; ++pr) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (dt < n_dt) {
-        const bf16x8 vf = SWZ ? ld16(vt + v_swz(16 * dt + r, 4 * pr + c)) : ld16(vt + (16 * dt + r) * v_stride + 32 * pr + 8 * c);
+    for (int dt = 0; dt < VD; ++dt) {
+      if (dt0 + dt < n_dt) {
+        const bf16x8 vf = SWZ ? ld16(vt + v_swz(16 * (dt0 + dt) + r, 4 * pr + c))
+                              : ld16(vt + (16 * (dt0 + dt) + r) * v_stride + 32 * pr + 8 * c);
 #pragma unroll
         for (int g = 0; g < QG; ++g) o[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[pr][g], o[g][dt], 0, 0, 0);
       }
@@ -303,11 +307,12 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 }
 
 // Runs the wave's 16 columns over tiles [tile_beg, tile_end) straight from the cache pages.
-template <int DT, bool EXACT, bool MOD>
-__device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
+template <int DT, bool EXACT, bool MOD, int VD = DT>
+__device__ __forceinline__ void attend(f32x4 (&o)[1][VD], float (&m_run)[1], float (&l_run)[1],
                                        const bf16x8 (&qf)[1][(DT + 1) / 2], const bf16_t* kh, const bf16_t* vh,
                                        const int* table, int page_size, int64_t page_stride, int hd, int tile_beg,
-                                       int tile_end, int p, bool valid, int lo_q, float scale2, const ColMod<1, MOD>& cm) {
+                                       int tile_end, int p, bool valid, int lo_q, float scale2, const ColMod<1, MOD>& cm,
+                                       int dt0 = 0) {
   const int pq[1] = {valid ? p : -1}, lq[1] = {lo_q};
   for (int tile = tile_beg; tile < tile_end; ++tile) {
     const int pos0 = tile * TILE;
@@ -316,7 +321,7 @@ __device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], flo
     const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
     const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
     const bool masked = pos0 + TILE - 1 > p || pos0 < lo_q;      // the same for all lanes
-    tile_step<DT, 1, EXACT, false, EXACT, MOD>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked, cm);
+    tile_step<DT, 1, EXACT, false, EXACT, MOD, VD>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked, cm, dt0);
   }
 }
 
@@ -593,11 +598,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
 // that no wave has more than one or two of them (left to the last wave alone, 30 runs in a row made a step with
 // one sequence beyond position 4096 and seven shorter ones a third slower).
 // AHEAD (with EXACT): the form for steps of few waves, which fetches a tile ahead (attend_ahead).
-template <int DT, bool EXACT, bool AHEAD = false, bool MOD = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD || DT > 16 ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
+// VS: the waves of a run that share a head's value dimensions among them (heads beyond 256: four, each with the scores of
+// the whole head and a quarter of the sums, so that a step has four times the waves and none holds 128 registers of sums).
+template <int DT, bool EXACT, bool AHEAD = false, bool MOD = false, int VS = 1>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
+  static_assert(DT % VS == 0 && (VS == 1 || !AHEAD), "the value dimensions are shared in whole blocks");
+  constexpr int VD = DT / VS;
   const int b = blockIdx.z;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
-  const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
+  const int dt0 = (int)(blockIdx.y % VS) * VD, y = blockIdx.y / VS;
+  const int kvh = y / ngc, cg = y % ngc;
   const int lane = threadIdx.x, r = lane % 16, c = lane / 16;
   const int p = a.start[b];
   const int lo = reach_lo(p, a.window, a.mod.chunk);
@@ -617,26 +627,26 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD || DT 
   for (int run = blockIdx.x; run < n_runs; run += gridDim.x) {
     const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
     if (tile_beg >= tile_end) continue;       // all of the run lies before the window
-    f32x4 o[1][DT];
+    f32x4 o[1][VD];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt < VD; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
     if constexpr (AHEAD)
       attend_ahead<DT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
                        tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm);
     else
-      attend<DT, EXACT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm);
+      attend<DT, EXACT, MOD, VD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm, dt0);
     if (!valid) continue;
     float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (16 * dt < a.hd) {
+    for (int dt = 0; dt < VD; ++dt) {
+      if (16 * (dt0 + dt) < a.hd) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[0][dt][v];
+        for (int v = 0; v < 4; ++v) out[16 * (dt0 + dt) + 4 * c + v] = o[0][dt][v];
       }
     }
-    if (c == 0) {
+    if (c == 0 && dt0 == 0) {
       out[a.hd] = m_run[0];
       out[a.hd + 1] = l_run[0];
     }
@@ -647,9 +657,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD || DT 
 // 2^(m_s - m) of the runs are worked out once, a lane per run, and kept in LDS; then every lane sums its
 // dimensions over the runs in order.
 #define MAX_RUNS_LDS 2048
-__global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
-  __shared__ float wgt[MAX_RUNS_LDS];
-  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+// (heads of 128, 256, 384 or 512: a wave to every 128 dimensions, each working out the weights for itself, so that no
+// wave waits for another)
+__global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
+  extern __shared__ float wgt_all[];        // [waves][MAX_RUNS_LDS]
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  float* wgt = wgt_all + wave * MAX_RUNS_LDS;
   const int p = a.start[b];
   const int lo = reach_lo(p, a.window, a.mod.chunk);
   const int S = tiles_per_run(p);
@@ -677,15 +690,16 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
   __builtin_amdgcn_wave_barrier();
   const float inv = 1.0f / l;
   bf16_t* orow = a.out + ((size_t)a.cu_seqlens[b] * a.nh + h) * a.hd;
-  if (a.hd == 128) {          // a lane takes two neighbouring dimensions: one pass over the runs, 8 bytes at a time
+  if (a.hd % 128 == 0) {      // a lane takes two neighbouring dimensions of its wave's 128: one pass over the runs, 8 bytes at a time
+    const int d = 128 * wave + 2 * lane;
     float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll 8
     for (int s = run_beg; s < run_end; ++s) {
-      const float2 v = *reinterpret_cast<const float2*>(part + (size_t)s * stride + 2 * lane);
+      const float2 v = *reinterpret_cast<const float2*>(part + (size_t)s * stride + d);
       acc0 = fmaf(wgt[s - run_beg], v.x, acc0);
       acc1 = fmaf(wgt[s - run_beg], v.y, acc1);
     }
-    *reinterpret_cast<uint32_t*>(orow + 2 * lane) = pack2(acc0 * inv, acc1 * inv);
+    *reinterpret_cast<uint32_t*>(orow + d) = pack2(acc0 * inv, acc1 * inv);
     return;
   }
   for (int d = lane; d < a.hd; d += 64) {
@@ -716,14 +730,19 @@ static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st)
 template <int DT, bool EXACT, bool MOD>
 static void launch_decode_as(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
   const int g = a.nh / a.nkv;
-  const dim3 grid(grid_runs, a.nkv * ((g + 15) / 16), B);
-  // at most a wave to a SIMD: each has the registers to fetch a tile ahead (one sequence at position 8,191: 2.38 ms a
-  // step against 2.61; with more waves than that the form is no faster, from twice as many on slower)
-  if (EXACT && DT <= 8 && (int64_t)grid.x * grid.y * grid.z <= 1024)
-    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, EXACT && DT <= 8, MOD>), grid, dim3(64), 0, st, a);
-  else
-    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, false, MOD>), grid, dim3(64), 0, st, a);
-  hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
+  const dim3 join_block(a.hd % 128 == 0 ? 64 * (a.hd / 128) : 64);      // a wave to every 128 dimensions of a head
+  if constexpr (DT > 16) {
+    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, false, MOD, 4>), dim3(grid_runs, a.nkv * ((g + 15) / 16) * 4, B), dim3(64), 0, st, a);
+  } else {
+    const dim3 grid(grid_runs, a.nkv * ((g + 15) / 16), B);
+    // at most a wave to a SIMD: each has the registers to fetch a tile ahead (one sequence at position 8,191: 2.38 ms a
+    // step against 2.61; with more waves than that the form is no faster, from twice as many on slower)
+    if (EXACT && DT <= 8 && (int64_t)grid.x * grid.y * grid.z <= 1024)
+      hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, EXACT && DT <= 8, MOD>), grid, dim3(64), 0, st, a);
+    else
+      hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, false, MOD>), grid, dim3(64), 0, st, a);
+  }
+  hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), join_block, join_block.x / 64 * MAX_RUNS_LDS * sizeof(float), st, a);
 }
 template <int DT, bool EXACT>
 static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
