@@ -450,6 +450,27 @@ def test_activation_rows_and_scaled_capped_logits():
         assert np.abs(t.double().cpu().numpy() - want).max() < 1e-5
 
 
+def test_a_product_whose_result_passes_an_activation():
+    """In the product's own epilogue (few rows, tiles) and behind the vendor's product (many rows), in both types."""
+    from turboquant_cpp_amd.csrc import ops
+    rng = np.random.default_rng(3)
+    for M, N, K in ((1, 96, 64), (8, 200, 128), (40, 136, 72), (300, 256, 264), (800, 128, 128)):
+        a = torch.tensor(rng.normal(size=(M, K)), dtype=torch.float32, device="cuda")
+        w = torch.tensor(rng.normal(size=(N, K)) * K ** -0.5, dtype=torch.float32, device="cuda")
+        bias = torch.tensor(rng.normal(size=(N,)), dtype=torch.float32, device="cuda")
+        for act, dt, tol in (("float32", torch.float32, 1e-4), ("bfloat16", torch.bfloat16, 0.04)):
+            aa, ww = a.to(dt), w.to(dt)
+            z = aa.double().cpu().numpy() @ ww.double().cpu().numpy().T
+            for name, f in (("relu2", lambda v: np.maximum(v, 0.0) ** 2), ("silu", plain.silu)):
+                got = ops.gemm(aa, ww, act, activation=name, act_alone=True)
+                assert got.dtype == dt and np.abs(got.double().cpu().numpy() - f(z)).max() < tol * max(1.0, np.abs(f(z)).max())
+            got = ops.gemm(aa, ww, act, bias=bias, activation="relu2", act_alone=True)
+            want = np.maximum(z + bias.double().cpu().numpy(), 0.0) ** 2
+            assert np.abs(got.double().cpu().numpy() - want).max() < tol * max(1.0, np.abs(want).max())
+            plain_product = ops.gemm(aa, ww, act)          # and nothing of it sticks to the next plain product
+            assert np.abs(plain_product.double().cpu().numpy() - z).max() < tol * max(1.0, np.abs(z).max())
+
+
 def test_delta_rule_kernels_with_a_state_carried_over(made):
     """The mixer's kernels against the plain function, the sequence cut in three runs so that each starts from the one
     before's state and convolution inputs, the last through the decode step's single kernel; two sequences side by side

@@ -16,6 +16,7 @@
 #define TQ_ERR_UNSUPPORTED (-2)
 // added to a tile_rows of 64 of a product over experts: two units of one expert per workgroup (see tq_gemm_mfma)
 #define TQ_TILE_PAIRS 1024
+#define TQ_GEMM_ACT_ALONE 256      // added to tq_gemm_mfma's gate: the activation of a plain product's result
 
 struct bf16_t {
   uint16_t bits;

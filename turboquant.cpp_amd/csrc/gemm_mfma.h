@@ -28,6 +28,7 @@ struct MfmaGemmArgs {
   int64_t split_stride;
   int gate;                 // activation of the gated pair
   int group_ratio;          // tile kernel: row tiles per entry of tile_group and unit of n_tiles (0 or 1: one)
+  int act1;                 // a plain product (no w2, k not split): 0, or 1 + the activation its result passes before it is stored
 };
 
 // For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on
@@ -58,6 +59,7 @@ __device__ __forceinline__ float bias_at(const MfmaGemmArgs& g, int n) {
 
 template <bool OUT_ACT>
 __device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, float v) {
+  if (g.act1) v = gate_fn(v, g.act1 - 1);
   if (OUT_ACT)
     ((bf16_t*)g.out)[(size_t)m * g.ldc + n] = f32_to_bf16(v);
   else

@@ -848,6 +848,8 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 // row tiles (tile_group[M / 64 ..], n_tiles[1]).
 // splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
 // the bias to run 0; the sum over the runs is the caller's.
+// gate: the activation of the gated pair; without w2 and with TQ_GEMM_ACT_ALONE added, the activation that the plain
+// product's result (bias included) passes before it is stored (a feed-forward of two matrices needs no launch between them).
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
                         int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
                         int bias_type, void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows,
@@ -856,12 +858,16 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0) return TQ_ERR_BAD_ARG;
   if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)w2) % 16 != 0 || (group_stride % 8) != 0) return TQ_ERR_BAD_ARG;
   const bool dual = w2 != nullptr, out_act = out_is_act != 0;
+  const bool alone = gate >= TQ_GEMM_ACT_ALONE;
+  if (alone) gate -= TQ_GEMM_ACT_ALONE;
   if (splits < 1 || splits > 64 || gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
+  if (alone && (dual || splits > 1)) return TQ_ERR_BAD_ARG;
   if (splits > 1 && (dual || out_act || tile_group || a_rows || splits != tq_gemm_mfma_splits(M, N, K))) return TQ_ERR_BAD_ARG;
   const int k_per = ((K + TBK - 1) / TBK + splits - 1) / splits * TBK;
   if (splits > 1 && (int64_t)(splits - 1) * k_per >= K) return TQ_ERR_BAD_ARG;
   MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
-                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate, 1};
+                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate, 1,
+                 alone ? gate + 1 : 0};
   int rc = 0;
   if (tile_group) {
     if (tile_rows == 16) {

@@ -758,9 +758,11 @@ def _use_f32(act, a: torch.Tensor, w: torch.Tensor, K: int, gstride: int) -> boo
 def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
          out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
          n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
-         partial_sums: bool = False, activation: str = "silu") -> torch.Tensor:
+         partial_sums: bool = False, activation: str = "silu", act_alone: bool = False) -> torch.Tensor:
     """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: f(a w^T) * (a w2^T), f being the
-    ``activation`` (silu, gelu_tanh or relu2).
+    ``activation`` (silu, gelu_tanh or relu2).  ``act_alone`` (a plain product, no ``w2``): f of the product, in the
+    activation type: in the product's own epilogue where this library's matrix-core kernel runs it, else in a launch
+    of its own behind it.
 
     ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
     ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
@@ -779,6 +781,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
               "partial sums are for plain products into float32")
     lib = library(act)
     gate = _gate_code(k, activation)
+    if act_alone:
+        _need(w2 is None and not partial_sums and not grouped and a_rows is None, k, "an activation alone is for plain products")
+        if (dtype_name(act) == "bfloat16" and not (bias is None and _vendor_product(act, a, w, M, K))
+                and _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE)):
+            out = torch.empty((M, N), dtype=adt, device=a.device)
+            _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), None, 1, _ptr(w), None, gstride, None, None, _ptr(bias),
+                                               _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, 1, M, N, K,
+                                               tile_rows, 1, gate + 256, _stream()))
+            return out
+        return act_rows(gemm(a, w, act, bias=bias), None, activation, act)
     if not grouped and a_rows is None and bias is None and _vendor_product(act, a, w, M, K):
         if w2 is None:
             out = _vendor_gemm(a, w, out_act)

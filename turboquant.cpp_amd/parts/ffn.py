@@ -75,7 +75,7 @@ class DenseActivated(Part):
                 "down": ParamSpec((self.hidden_size, self.inner_size))}
 
     def forward(self, normed, normed32, ctx):
-        h = ops.act_rows(ops.gemm(normed, self.up, ctx.act), None, self.activation, ctx.act)
+        h = ops.gemm(normed, self.up, ctx.act, activation=self.activation, act_alone=True)
         return ops.gemm(h, self.down, ctx.act, partial_sums=True)
 
 
