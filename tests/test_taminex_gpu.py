@@ -412,7 +412,8 @@ def test_products_per_head_with_a_gate_and_the_latent_s_norm():
     from turboquant_cpp_amd.csrc import ops
     rng = np.random.default_rng(1)
     f32 = lambda a: torch.tensor(np.ascontiguousarray(a), dtype=torch.float32, device="cuda")
-    for T, H, N, K in ((1, 3, 20, 12), (37, 2, 48, 32), (130, 5, 16, 304), (300, 4, 128, 64)):
+    for T, H, N, K in ((1, 3, 20, 12), (37, 2, 48, 32), (130, 5, 16, 304), (300, 4, 128, 64), (1, 4, 128, 512), (8, 3, 520, 128),
+                       (16, 2, 24, 40), (5, 2, 16, 264)):
         a, wt, g = rng.normal(size=(T, H * K)), rng.normal(size=(H, N, K)), rng.normal(size=(T, H * N))
         want = np.einsum("thk,hnk->thn", a.reshape(T, H, K), wt).reshape(T, H * N)
         wide = f32(np.concatenate([rng.normal(size=(T, 5)), a, rng.normal(size=(T, 3))], axis=1))     # a run of columns

@@ -7,12 +7,13 @@
 // activation type with a row stride of its own, so that it can be a run of columns of a wider product; `out` likewise.
 // The epilogue can multiply by f(gate[t][h N + n]), f an activation of gates.def: an output gate costs no pass of its own.
 //
-// Two kernels.  bfloat16 library, bfloat16 matrices, K a multiple of 8: v_mfma_f32_16x16x32_bf16 with both operands
+// Three kernels.  bfloat16 library, bfloat16 matrices, K a multiple of 8: v_mfma_f32_16x16x32_bf16 with both operands
 // straight from memory, 16 bytes per lane (the first operand is 16 rows n of the head's matrix, the second 16 tokens,
 // so that a lane ends up with four neighbouring n of one token and stores them as one piece); a wave owns 32 tokens by
 // 64 n, and a head's matrix is a few hundred KB at most, which the caches keep while the tokens pass.  Everything
 // else: a tile of 64 tokens by 64 n per workgroup, staged through LDS in steps of 16 k, plain multiply-adds in float.
-// Both sum over k in ascending order whatever the number of tokens.
+// (up to 16 tokens: a wave owns 16 tokens by 16 n and has eight steps of k in flight, head_gemm_few_kernel).
+// All sum over k in ascending order whatever the number of tokens.
 #include "common.h"
 
 struct HeadGemmArgs {
@@ -158,6 +159,41 @@ __global__ __launch_bounds__(256) void head_gemm_mfma_kernel(HeadGemmArgs g, int
       }
   }
 }
+
+// A step of few tokens (a decode step): a wave takes 16 tokens by 16 n, so that a head's matrix is spread over eight times
+// the waves of the kernel above, and fetches eight steps of k from clamped addresses before it multiplies any, so that
+// the loads are in flight together (K = 512: two rounds of loads instead of sixteen).
+template <class A, bool OUT_ACT>
+__global__ __launch_bounds__(256) void head_gemm_few_kernel(HeadGemmArgs g, int n_tiles, int items) {
+  const int id = blockIdx.x * 4 + threadIdx.x / 64;
+  if (id >= items) return;
+  const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+  const int t0 = id / n_tiles * 16, n0 = id % n_tiles * 16, h = blockIdx.z;
+  const A* arow = (const A*)g.a + (size_t)h * g.K + (size_t)min(t0 + r, g.T - 1) * g.lda;
+  const bf16_t* wrow = (const bf16_t*)g.w + ((size_t)h * g.N + min(n0 + r, g.N - 1)) * g.K;
+  hg_f32x4 acc = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < g.K; k0 += 256) {
+    hg_bf16x8 af[8], wf[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = min(k0 + 32 * s + 8 * c, g.K - 8);
+      af[s] = hg_load8(arow + k);
+      wf[s] = hg_load8(wrow + k);
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (k0 + 32 * s + 8 * c >= g.K) af[s] = hg_zero8();        // a step past the end adds nothing
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af[s], acc, 0, 0, 0);
+    }
+  }
+  const int t = t0 + r;
+  if (t >= g.T) return;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int n = n0 + 4 * c + v;
+    if (n < g.N) hg_store<OUT_ACT>(g, t, h * g.N + n, acc[v]);
+  }
+}
 #endif
 
 // a [T][>= H K] of a_type (TQ_F32, or TQ_BF16 on the bfloat16 library) with row stride lda; w [H][N][K] of wtype;
@@ -176,6 +212,20 @@ TQ_API int tq_head_gemm(const void* a, int a_type, int64_t lda, const void* w, i
 #if defined(TQ_ACT_BF16)
   const bool a_f32 = a_type == TQ_F32;
   if (wtype == TQ_BF16 && K % 8 == 0 && lda % (a_f32 ? 4 : 8) == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0) {
+    if (T <= 16) {
+      const int n16 = (N + 15) / 16;
+      const dim3 grid_few((unsigned)((n16 + 3) / 4), 1, H);
+#define TQ_HG_FEW(AT)                                                                                               \
+  do {                                                                                                              \
+    if (out_act) hipLaunchKernelGGL((head_gemm_few_kernel<AT, true>), grid_few, dim3(256), 0, st, g, n16, n16);     \
+    else hipLaunchKernelGGL((head_gemm_few_kernel<AT, false>), grid_few, dim3(256), 0, st, g, n16, n16);            \
+  } while (0)
+      if (a_f32) TQ_HG_FEW(float);
+      else TQ_HG_FEW(bf16_t);
+#undef TQ_HG_FEW
+      TQ_LAUNCH_CHECK();
+      return 0;
+    }
     const int n_tiles = (N + 63) / 64;
     const int64_t items = (int64_t)((T + 31) / 32) * n_tiles;
     if (items > (int64_t)4 * 2147483647) return TQ_ERR_UNSUPPORTED;
