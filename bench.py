@@ -294,7 +294,7 @@ def taminex_config(z: dict, layers: int, max_positions: int) -> dict:
             layer["mixer"]["kv_from"] = i - 1
         out.append(layer)
     return {"architecture": "Taminex", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
-            "logit_softcap": 30.0, "layers": out}
+            "logit_softcap": 40.0, "layers": out}
 
 
 def qwen_dense_config_like(z: dict, layers: int, max_positions: int) -> dict:

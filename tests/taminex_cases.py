@@ -84,12 +84,12 @@ CASES = {
     ], logit_softcap=20.0),
     # as a served model's layers might be laid out, small
     "regular": config(128, 256, [
-        (delta(4, 2, 32, 32), dense(256)),
-        (attention(4, 1, 64, 64, rot=32, base=1e5), dense(256)),
-        (delta(4, 4, 32, 64), dense(256)),
-        (latent(4, 32, 32, 64), dense(256)),
-        (latent(4, 32, 32, 64, kv_from=3), dense(256)),
-    ], logit_scale=2.0, logit_softcap=30.0),
+        (delta(4, 2, 32, 48), dense(192)),
+        (attention(4, 1, 64, 64, rot=16, base=1e5), dense(192)),
+        (delta(4, 4, 32, 64), dense(320)),
+        (latent(4, 32, 32, 64), dense(192)),
+        (latent(4, 32, 32, 64, kv_from=3), dense(320)),
+    ], logit_scale=1.5, logit_softcap=24.0),
 }
 
 

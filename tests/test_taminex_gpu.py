@@ -425,7 +425,7 @@ def test_products_per_head_with_a_gate_and_the_latent_s_norm():
         got = ops.head_gemm(f32(a).bfloat16(), f32(wt).bfloat16(), "bfloat16", out_act=True, gate=f32(g), activation="sigmoid")
         assert got.dtype == torch.bfloat16
         assert np.abs(got.double().cpu().numpy() - want * plain.sigmoid(g)).max() < 0.03 * np.abs(want).max()
-    for T, R, width, copies in ((1, 20, 32, 2), (70, 96, 96, 2), (9, 304, 304, 1), (33, 18, 32, 3)):
+    for T, R, width, copies in ((1, 20, 32, 2), (70, 80, 80, 2), (9, 304, 304, 1), (33, 18, 32, 3)):
         src, wt = rng.normal(size=(T, R + 7)), rng.normal(1, 0.1, R)
         out = torch.full((T, copies * width + 2), 7.0, dtype=torch.float32, device="cuda")
         ops.latent_norm(f32(src)[:, 3:3 + R], f32(wt), 1e-5, out[:, 1:1 + copies * width], copies, width, "float32")
@@ -444,7 +444,7 @@ def test_activation_rows_and_scaled_capped_logits():
     zg = torch.tensor(z, dtype=torch.float32, device="cuda")
     got = ops.act_rows(zg, None, "relu2", "float32")
     assert np.abs(got.double().cpu().numpy() - np.maximum(z, 0.0) ** 2).max() < 1e-5
-    for scale, cap in ((2.0, 30.0), (0.5, None), (1.0, 4.0), (3.0, 1.5)):
+    for scale, cap in ((2.5, 20.0), (0.5, None), (1.0, 4.0), (3.0, 1.5)):
         t = zg.clone()
         ops.softcap(t, cap, "float32", scale=scale)
         want = z * scale if cap is None else cap * np.tanh(z * scale / cap)

@@ -204,7 +204,7 @@ _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pa
          "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
          "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
          "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn",
-         "head_gemm": "matmul", "latent_norm": "attn"}
+         "head_gemm": "matmul", "latent_norm": "attn", "gate_rows": "attn"}
 
 
 def profile_begin() -> None:
