@@ -5,7 +5,7 @@ own that would expand it, k_h = W_uk,h c and v_h = W_uv,h c; the score of query 
 (q_h,i . k_h,j) * scale, the softmax is the ordinary one, the concatenated heads are multiplied element by element by
 sigmoid(W_g x) and go through the output product.
 
-The keys and values are never expanded.  Since q . (W_uk c) = (W_uk^T q) . c, each head's key matrix is folded into its
+In the folded form the keys and values are never expanded.  Since q . (W_uk c) = (W_uk^T q) . c, each head's key matrix is folded into its
 query (one product per head, ``ops.head_gemm``), and since sum_j p_j W_uv c_j = W_uv sum_j p_j c_j, each head's value
 matrix is applied to its weighted sum of latents afterwards (a second product per head, whose epilogue applies the output
 gate).  In between runs the library's attention over the paged cache as for any mixer with one key/value head shared by
@@ -14,7 +14,7 @@ and in the cache): the cache holds the latent as a key row and, transposed, as a
 attention kernels' operands take.  Decoded tokens and portions of prompts that go on from earlier tokens take this form:
 it reads ``kv_rank`` numbers per position whatever the number of heads.
 
-A step whose sequences all start at their first token takes the other form, since per pair of positions the folded form
+A step whose sequences all start at their first token takes the other, expanded form, since per pair of positions the folded form
 costs heads x 2 ``kv_rank`` multiply-adds and the expanded one heads x (dim + vdim): one product expands the step's
 latents into every head's keys and values, which are laid into pages that live for the step only
 (``StepBatch.own_pages``), and the library's attention runs over them with as many key/value heads as heads; the output
